@@ -1,0 +1,138 @@
+/*
+ * segpt_attn.h -- C ABI of libsegpt_attn.so: fused QK-norm causal GQA flash
+ * attention (forward + backward) for AMD MI355X (gfx950).
+ *
+ * The library is the device side of a drop-in for the reference's fused op
+ *   sample_efficient_gpt/transformer/ops/triton_flash_attn_qknorm.py:262-343
+ *   (TritonFlashAttnQKNormFunc) and of the live module it stands in for
+ *   sample_efficient_gpt/transformer/attention.py:43-80 (SelfDotProductAttnQKNorm),
+ * plus the caller glue the kernels absorb (GQA expansion attention.py:207-218,
+ * value-residual mix :222-228, per-head gate :249-255).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; no torch / HIP types in any signature
+ *     (`stream` is a hipStream_t passed as void*; NULL = the null stream);
+ *   - the caller owns ALL memory (inputs, outputs, workspace); the library never
+ *     allocates, frees or keeps device pointers past a call, and never
+ *     synchronises: work is enqueued on `stream` and the call returns;
+ *   - return value: 0 ok; < 0 argument / unsupported-shape error detected before
+ *     any launch (SEGPT_E_*); > 0 a hipError_t raised by a launch;
+ *   - re-entrant: no mutable global state.
+ *
+ * Mathematics (per batch b, query head h, kv head g = h / (H/Hkv)):
+ *   a_i = rsqrt(mean_d q_i^2 + eps)      b_j = rsqrt(mean_d k_j^2 + eps)
+ *   s_ij = sm_scale * sum_d (a_i q_id g_q[d]) (b_j k_jd g_k[d]),  j <= i + q_start if causal
+ *   v'_j = c1 v_j + c2 v_first_j         (if vr_coef != NULL, (c1,c2) = vr_coef[0..1])
+ *   lse_i = log sum_j exp s_ij ;  o_i = sum_j exp(s_ij - lse_i) v'_j
+ *   y_i = gate_scale * sigmoid(gate[b,i,h]) * o_i   (if gate.ptr != NULL; else y = o)
+ * With g_q = gain (1 element), g_k absent, eps = 1e-6, sm_scale = 1/sqrt(D) this is
+ * attention.py:51-80; eps = 1e-8/D, sm_scale = 1/D gives triton_flash_attn_qknorm.py:67-91.
+ */
+#ifndef SEGPT_ATTN_H
+#define SEGPT_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SEGPT_ABI_VERSION 1
+
+/* element type of q/k/v/o/gate and their gradients */
+#define SEGPT_DTYPE_BF16 0 /* MFMA path: D in {64, 128}                       */
+#define SEGPT_DTYPE_FP32 1 /* fp32 FMA path (1e-5 parity): D in {32, 64, 128} */
+
+/* error codes (negative); segpt_strerror() gives the text */
+#define SEGPT_OK 0
+#define SEGPT_E_NULL -1        /* a required pointer is NULL                                */
+#define SEGPT_E_STRUCT -2      /* struct_bytes does not match this library's layout         */
+#define SEGPT_E_DTYPE -3       /* unknown dtype                                             */
+#define SEGPT_E_SHAPE -4       /* B,H,Hkv,Sq,Sk <= 0, H % Hkv != 0, or numel of a scale     */
+#define SEGPT_E_HEAD_DIM -5    /* D not supported for this dtype                            */
+#define SEGPT_E_STRIDE -6      /* a stride is negative / misaligned (rows must be 16 B aligned) */
+#define SEGPT_E_WORKSPACE -7   /* workspace NULL or smaller than segpt_attn_workspace_bytes */
+#define SEGPT_E_EXTRAS -8      /* v_first without vr_coef or the reverse; missing grad slot */
+#define SEGPT_E_QSTART -9      /* q_start < 0                                               */
+#define SEGPT_E_ALIGN -10      /* a base pointer is not 16-byte aligned                     */
+
+/* [B, heads, S, D] tensor view; the D axis is contiguous (stride 1). Strides in ELEMENTS.
+ * The reference's `(h b) S D` flatten (attention.py:199) is stride_b = S*D, stride_h = B*S*D;
+ * a `b S (h D)` projection slice is stride_b = S*W, stride_h = D, stride_s = W. */
+typedef struct segpt_tensor4 {
+  void* ptr;
+  int64_t stride_b, stride_h, stride_s;
+} segpt_tensor4;
+
+/* [B, Sq, H] per-head gate logits view (attention.py:251: attn_gate(x) is `b seq h`). */
+typedef struct segpt_tensor3 {
+  void* ptr;
+  int64_t stride_b, stride_s, stride_h;
+} segpt_tensor3;
+
+typedef struct segpt_attn_params {
+  uint32_t struct_bytes; /* = sizeof(segpt_attn_params) */
+  int32_t dtype;         /* SEGPT_DTYPE_* */
+  int32_t B, H, Hkv, Sq, Sk, D;
+  int32_t causal;  /* 0 / 1 */
+  int32_t q_start; /* causal diagonal shift: key j visible to query i iff j <= i + q_start */
+  int32_t gq_numel; /* 1 (scalar gain, attention.py:41) or D */
+  int32_t gk_numel; /* 0 (no k scale), 1 or D */
+  float eps, sm_scale, gate_scale;
+  int32_t reserved0;
+
+  /* forward operands */
+  segpt_tensor4 q;       /* [B,H,Sq,D]   in  */
+  segpt_tensor4 k;       /* [B,Hkv,Sk,D] in  */
+  segpt_tensor4 v;       /* [B,Hkv,Sk,D] in  */
+  segpt_tensor4 v_first; /* [B,Hkv,Sk,D] in, optional (ptr NULL = no value residual) */
+  segpt_tensor3 gate;    /* [B,Sq,H]     in, optional (ptr NULL = no gate) */
+  segpt_tensor4 o;       /* [B,H,Sq,D]   fwd: out (y, gated if gate);  bwd: in (the saved y) */
+  float* lse;            /* [B,H,Sq] contiguous fp32, natural log; fwd: out, bwd: in */
+  const float* g_q;      /* [gq_numel] fp32 device */
+  const float* g_k;      /* [gk_numel] fp32 device or NULL */
+  const float* vr_coef;  /* [2] fp32 device (c1, c2) or NULL */
+
+  /* backward operands (ignored by segpt_attn_fwd) */
+  segpt_tensor4 d_o;      /* [B,H,Sq,D]   in: dL/dy */
+  segpt_tensor4 dq;       /* [B,H,Sq,D]   out */
+  segpt_tensor4 dk;       /* [B,Hkv,Sk,D] out */
+  segpt_tensor4 dv;       /* [B,Hkv,Sk,D] out */
+  segpt_tensor4 dv_first; /* [B,Hkv,Sk,D] out, required iff v_first */
+  segpt_tensor3 dgate;    /* [B,Sq,H]     out, required iff gate */
+  float* dg_q;            /* [gq_numel] fp32 out */
+  float* dg_k;            /* [gk_numel] fp32 out, required iff g_k */
+  float* dvr_coef;        /* [2] fp32 out, required iff vr_coef */
+
+  void* workspace; /* >= segpt_attn_workspace_bytes(), 256 B aligned; contents undefined on entry */
+  size_t workspace_bytes;
+} segpt_attn_params;
+
+/* ABI revision of the loaded library (compare with SEGPT_ABI_VERSION). No reference counterpart. */
+int segpt_abi_version(void);
+
+/* Static text for a return code of this library (negative) or "hip error" class (positive).
+ * Replaces the Python AssertionErrors of triton_flash_attn_qknorm.py:273-276. */
+const char* segpt_strerror(int code);
+
+/* Bytes of device scratch the call needs (0 is possible for forward). Validates nothing but
+ * sizes; returns 0 for invalid params (the launch call will report the error).
+ * Replaces the in-op allocations of triton_flash_attn_qknorm.py:286-287 / :320-323: the caller
+ * allocates. */
+size_t segpt_attn_workspace_bytes(const segpt_attn_params* p, int is_bwd);
+
+/* Forward: writes o (y) and lse.  Replaces the launch
+ * `flashatt_qknorm_kernel_fwd[grid](...)`, triton_flash_attn_qknorm.py:290-302 (kernel :22-115),
+ * and in the live path the normalise + SDPA sequence attention.py:52-80. */
+int segpt_attn_fwd(const segpt_attn_params* p, void* stream);
+
+/* Backward: reads q,k,v,(v_first,gate),o,lse,d_o; writes dq,dk,dv,(dv_first,dgate),dg_q,(dg_k,dvr_coef).
+ * Deterministic (no floating-point atomics).  Replaces the launch
+ * `flashatt_qknorm_kernel_bwd[grid](...)`, triton_flash_attn_qknorm.py:326-342 (kernel :125-255). */
+int segpt_attn_bwd(const segpt_attn_params* p, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SEGPT_ATTN_H */

@@ -1,0 +1,15 @@
+"""MI355X-native fused QK-norm causal GQA flash attention (forward + backward).
+
+Drop-in for the attention hot path of thepowerfuldeez/sample_efficient_gpt:
+``QKNormFlashAttnFunc`` mirrors the reference's ``TritonFlashAttnQKNormFunc`` call signature,
+``SelfDotProductAttnQKNorm`` mirrors the live module, ``qknorm_attention`` is the same op on
+canonical ``[B, H, S, D]`` views.  All compute runs in hand-written HIP kernels (gfx950) reached
+through the C ABI of ``libsegpt_attn.so``; there is no fallback path.
+"""
+
+from .function import QKNormFlashAttnFunc, qknorm_attention  # noqa: F401
+from .module import SelfDotProductAttnQKNorm  # noqa: F401
+from .inputs import CONFIGS, AttnConfig, make_inputs  # noqa: F401
+
+# the reference's class name, so `from ... import TritonFlashAttnQKNormFunc` call sites keep working
+TritonFlashAttnQKNormFunc = QKNormFlashAttnFunc

@@ -1,0 +1,170 @@
+// C ABI of libsegpt_attn.so: argument validation, workspace carve-up and dispatch.
+// No device memory is allocated or freed here; nothing synchronises.
+#include "common.hpp"
+
+namespace segpt {
+
+int f32_rows_per_block();
+int bf16_dq_rows_per_block(int D);
+int bf16_dkdv_rows_per_block(int D);
+
+int dq_blocks(const segpt_attn_params& p) {
+  const int rows = p.dtype == SEGPT_DTYPE_FP32 ? f32_rows_per_block() : bf16_dq_rows_per_block(p.D);
+  return ((p.Sq + rows - 1) / rows) * p.H * p.B;
+}
+int dkdv_blocks(const segpt_attn_params& p) {
+  const int rows = p.dtype == SEGPT_DTYPE_FP32 ? f32_rows_per_block() : bf16_dkdv_rows_per_block(p.D);
+  return ((p.Sk + rows - 1) / rows) * p.Hkv * p.B;
+}
+
+namespace {
+
+size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
+size_t elem_bytes(const segpt_attn_params& p) { return p.dtype == SEGPT_DTYPE_FP32 ? 4 : 2; }
+
+struct WsLayout {
+  size_t delta, do_eff, dg_part, dcoef_part, total;
+};
+
+WsLayout bwd_layout(const segpt_attn_params& p) {
+  WsLayout w;
+  size_t off = 0;
+  const size_t rows = (size_t)p.B * p.H * p.Sq;
+  w.delta = off;
+  off += align_up(rows * sizeof(float));
+  w.do_eff = off;
+  if (p.gate.ptr) off += align_up(rows * p.D * elem_bytes(p));
+  w.dg_part = off;
+  off += align_up((size_t)dq_blocks(p) * p.D * sizeof(float));
+  w.dcoef_part = off;
+  off += align_up((size_t)dkdv_blocks(p) * 2 * sizeof(float));
+  w.total = off;
+  return w;
+}
+
+bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+int check_t4(const segpt_tensor4& t, const segpt_attn_params& p) {
+  if (!t.ptr) return SEGPT_E_NULL;
+  if (!aligned16(t.ptr)) return SEGPT_E_ALIGN;
+  const int64_t per16 = 16 / (int64_t)elem_bytes(p);
+  if (t.stride_b < 0 || t.stride_h < 0 || t.stride_s < p.D) return SEGPT_E_STRIDE;
+  if (t.stride_b % per16 || t.stride_h % per16 || t.stride_s % per16) return SEGPT_E_STRIDE;
+  return SEGPT_OK;
+}
+
+int check_common(const segpt_attn_params* p) {
+  if (!p) return SEGPT_E_NULL;
+  if (p->struct_bytes != sizeof(segpt_attn_params)) return SEGPT_E_STRUCT;
+  if (p->dtype != SEGPT_DTYPE_BF16 && p->dtype != SEGPT_DTYPE_FP32) return SEGPT_E_DTYPE;
+  if (p->B <= 0 || p->H <= 0 || p->Hkv <= 0 || p->Sq <= 0 || p->Sk <= 0) return SEGPT_E_SHAPE;
+  if (p->H % p->Hkv != 0) return SEGPT_E_SHAPE;
+  if (p->B > 65535 || p->H > 65535) return SEGPT_E_SHAPE;
+  if (p->dtype == SEGPT_DTYPE_BF16) {
+    if (p->D != 64 && p->D != 128) return SEGPT_E_HEAD_DIM;
+  } else {
+    if (p->D != 32 && p->D != 64 && p->D != 128) return SEGPT_E_HEAD_DIM;
+  }
+  if (p->gq_numel != 1 && p->gq_numel != p->D) return SEGPT_E_SHAPE;
+  if (p->gk_numel != 0 && p->gk_numel != 1 && p->gk_numel != p->D) return SEGPT_E_SHAPE;
+  if (p->q_start < 0) return SEGPT_E_QSTART;
+  if (!p->g_q || !p->lse) return SEGPT_E_NULL;
+  if ((p->gk_numel != 0) != (p->g_k != nullptr)) return SEGPT_E_SHAPE;
+  if ((p->v_first.ptr != nullptr) != (p->vr_coef != nullptr)) return SEGPT_E_EXTRAS;
+  int rc;
+  if ((rc = check_t4(p->q, *p))) return rc;
+  if ((rc = check_t4(p->k, *p))) return rc;
+  if ((rc = check_t4(p->v, *p))) return rc;
+  if ((rc = check_t4(p->o, *p))) return rc;
+  if (p->v_first.ptr && (rc = check_t4(p->v_first, *p))) return rc;
+  if (p->gate.ptr && (p->gate.stride_b < 0 || p->gate.stride_s < 0 || p->gate.stride_h < 0)) return SEGPT_E_STRIDE;
+  return SEGPT_OK;
+}
+
+int check_bwd(const segpt_attn_params* p) {
+  int rc;
+  if ((rc = check_t4(p->d_o, *p))) return rc;
+  if ((rc = check_t4(p->dq, *p))) return rc;
+  if ((rc = check_t4(p->dk, *p))) return rc;
+  if ((rc = check_t4(p->dv, *p))) return rc;
+  if (!p->dg_q) return SEGPT_E_NULL;
+  if (p->g_k && !p->dg_k) return SEGPT_E_EXTRAS;
+  if (p->v_first.ptr) {
+    if (!p->dv_first.ptr || !p->dvr_coef) return SEGPT_E_EXTRAS;
+    if ((rc = check_t4(p->dv_first, *p))) return rc;
+  }
+  if (p->gate.ptr) {
+    if (!p->dgate.ptr) return SEGPT_E_EXTRAS;
+    if (p->dgate.stride_b < 0 || p->dgate.stride_s < 0 || p->dgate.stride_h < 0) return SEGPT_E_STRIDE;
+  }
+  const WsLayout w = bwd_layout(*p);
+  if (!p->workspace || p->workspace_bytes < w.total) return SEGPT_E_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(p->workspace) & 255u) return SEGPT_E_ALIGN;
+  return SEGPT_OK;
+}
+
+}  // namespace
+}  // namespace segpt
+
+using namespace segpt;
+
+extern "C" {
+
+int segpt_abi_version(void) { return SEGPT_ABI_VERSION; }
+
+const char* segpt_strerror(int code) {
+  switch (code) {
+    case SEGPT_OK: return "ok";
+    case SEGPT_E_NULL: return "a required pointer is NULL";
+    case SEGPT_E_STRUCT: return "segpt_attn_params.struct_bytes does not match this library (ABI mismatch)";
+    case SEGPT_E_DTYPE: return "unknown dtype (expected SEGPT_DTYPE_BF16 or SEGPT_DTYPE_FP32)";
+    case SEGPT_E_SHAPE: return "bad shape: sizes must be positive, H divisible by Hkv, scale vectors of 1 or D elements";
+    case SEGPT_E_HEAD_DIM: return "unsupported head_dim: bf16 needs D in {64,128}, fp32 D in {32,64,128}";
+    case SEGPT_E_STRIDE: return "bad stride: strides must be non-negative multiples of 16 bytes and rows must not overlap";
+    case SEGPT_E_WORKSPACE: return "workspace missing or smaller than segpt_attn_workspace_bytes()";
+    case SEGPT_E_EXTRAS: return "inconsistent optional operands (v_first/vr_coef/gate and their gradient slots)";
+    case SEGPT_E_QSTART: return "q_start must be >= 0";
+    case SEGPT_E_ALIGN: return "a base pointer is not 16-byte aligned (workspace: 256-byte)";
+    default: return code > 0 ? "HIP runtime error raised by a kernel launch" : "unknown segpt error code";
+  }
+}
+
+size_t segpt_attn_workspace_bytes(const segpt_attn_params* p, int is_bwd) {
+  if (!p || p->struct_bytes != sizeof(segpt_attn_params)) return 0;
+  if (p->B <= 0 || p->H <= 0 || p->Hkv <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0) return 0;
+  if (!is_bwd) return 0;
+  if (p->dtype == SEGPT_DTYPE_BF16 && p->D != 64 && p->D != 128) return 0;
+  return bwd_layout(*p).total;
+}
+
+int segpt_attn_fwd(const segpt_attn_params* p, void* stream) {
+  int rc = check_common(p);
+  if (rc) return rc;
+  KArgs a{};
+  a.p = *p;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  return p->dtype == SEGPT_DTYPE_FP32 ? launch_fwd_f32(a, st) : launch_fwd_bf16(a, st);
+}
+
+int segpt_attn_bwd(const segpt_attn_params* p, void* stream) {
+  int rc = check_common(p);
+  if (rc) return rc;
+  if ((rc = check_bwd(p))) return rc;
+  const WsLayout w = bwd_layout(*p);
+  KArgs a{};
+  a.p = *p;
+  char* ws = reinterpret_cast<char*>(p->workspace);
+  a.delta = reinterpret_cast<float*>(ws + w.delta);
+  a.do_eff = p->gate.ptr ? ws + w.do_eff : nullptr;
+  a.dg_part = reinterpret_cast<float*>(ws + w.dg_part);
+  a.dcoef_part = reinterpret_cast<float*>(ws + w.dcoef_part);
+  a.n_dq_blocks = dq_blocks(*p);
+  a.n_dkdv_blocks = dkdv_blocks(*p);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if ((rc = launch_bwd_pre(a, st))) return rc;
+  rc = p->dtype == SEGPT_DTYPE_FP32 ? launch_bwd_f32(a, st) : launch_bwd_bf16(a, st);
+  if (rc) return rc;
+  return launch_bwd_reduce(a, st);
+}
+
+}  // extern "C"

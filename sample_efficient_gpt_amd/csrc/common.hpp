@@ -1,0 +1,105 @@
+// Shared device/host definitions for libsegpt_attn.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "segpt_attn.h"
+
+namespace segpt {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Everything a kernel needs: the caller's params by value plus the carved-up workspace.
+struct KArgs {
+  segpt_attn_params p;
+  float* delta;       // [B,H,Sq] fp32: rowsum(dO_eff * o)
+  void* do_eff;       // [B,H,Sq,D] dtype, contiguous: gate-scaled dO (only when gated)
+  float* dg_part;     // [n_dq_blocks, D] fp32 partial sums of the combined scale gradient
+  float* dcoef_part;  // [n_dkdv_blocks, 2] fp32 partial sums of (dc1, dc2)
+  int32_t n_dq_blocks;
+  int32_t n_dkdv_blocks;
+};
+
+struct __attribute__((aligned(16))) bf16x8_raw {
+  uint32_t w[4];
+};
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+
+// round-to-nearest-even fp32 -> bf16 (inputs are finite in every use below)
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  f2 v = {lo, hi};
+  bf2 r = __builtin_convertvector(v, bf2);  // v_cvt_pk_bf16_f32 on gfx950 (RNE)
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ float bf16lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+template <typename T>
+struct Elem;
+template <>
+struct Elem<float> {
+  static constexpr int kVec = 4;  // elements per 16-byte access
+  static __device__ __forceinline__ void load(const float* p, float (&out)[4]) {
+    float4 v = *reinterpret_cast<const float4*>(p);
+    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&in)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(in[0], in[1], in[2], in[3]);
+  }
+  static __device__ __forceinline__ float load1(const float* p) { return *p; }
+  static __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+};
+template <>
+struct Elem<uint16_t> {  // bf16 bits
+  static constexpr int kVec = 8;
+  static __device__ __forceinline__ void load(const uint16_t* p, float (&out)[8]) {
+    uint4 v = *reinterpret_cast<const uint4*>(p);
+    out[0] = bf16lo(v.x); out[1] = bf16hi(v.x); out[2] = bf16lo(v.y); out[3] = bf16hi(v.y);
+    out[4] = bf16lo(v.z); out[5] = bf16hi(v.z); out[6] = bf16lo(v.w); out[7] = bf16hi(v.w);
+  }
+  static __device__ __forceinline__ void store(uint16_t* p, const float (&in)[8]) {
+    uint4 v;
+    v.x = pack_bf16x2(in[0], in[1]); v.y = pack_bf16x2(in[2], in[3]);
+    v.z = pack_bf16x2(in[4], in[5]); v.w = pack_bf16x2(in[6], in[7]);
+    *reinterpret_cast<uint4*>(p) = v;
+  }
+  static __device__ __forceinline__ float load1(const uint16_t* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ void store1(uint16_t* p, float v) { *p = f32_to_bf16(v); }
+};
+
+template <typename T>
+__device__ __forceinline__ const T* row_ptr(const segpt_tensor4& t, int b, int h, int s) {
+  return reinterpret_cast<const T*>(t.ptr) + (int64_t)b * t.stride_b + (int64_t)h * t.stride_h + (int64_t)s * t.stride_s;
+}
+template <typename T>
+__device__ __forceinline__ T* row_ptr_mut(const segpt_tensor4& t, int b, int h, int s) {
+  return reinterpret_cast<T*>(t.ptr) + (int64_t)b * t.stride_b + (int64_t)h * t.stride_h + (int64_t)s * t.stride_s;
+}
+
+__device__ __forceinline__ float sigmoidf_acc(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// host-side launchers (one per translation unit); each returns a hipError_t as int
+int launch_fwd_f32(const KArgs& a, hipStream_t st);
+int launch_bwd_f32(const KArgs& a, hipStream_t st);
+int launch_fwd_bf16(const KArgs& a, hipStream_t st);
+int launch_bwd_bf16(const KArgs& a, hipStream_t st);
+int launch_bwd_pre(const KArgs& a, hipStream_t st);     // delta, dgate, do_eff
+int launch_bwd_reduce(const KArgs& a, hipStream_t st);  // dg_q, dg_k, dvr_coef from the partials
+
+// block counts shared by the workspace carve-up and the launchers
+int dq_blocks(const segpt_attn_params& p);
+int dkdv_blocks(const segpt_attn_params& p);
+
+}  // namespace segpt

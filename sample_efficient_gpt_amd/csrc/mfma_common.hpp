@@ -1,0 +1,193 @@
+// Building blocks shared by the bf16 MFMA kernels (gfx950, wave64).
+//
+// MFMA used everywhere: v_mfma_f32_32x32x16_bf16, D(32x32) += A(32x16) * B(16x32).
+//   A operand, lane l: row  = l % 32, k = 8*(l/32) + t, t = 0..7   (8 bf16 = 4 VGPRs)
+//   B operand, lane l: col  = l % 32, k = 8*(l/32) + t
+//   C/D,       lane l: col  = l % 32, row(r) = 8*(r/4) + 4*(l/32) + r%4, r = 0..15
+// A C tile whose rows are the contraction index of the next product is reused directly as that
+// product's B (or A) operand: registers 8s..8s+7 of a lane hold rows {4hh..4hh+3, 8+4hh..8+4hh+3} + 16s
+// (hh = l/32).  The contraction order inside an MFMA is free as long as both operands agree, so the
+// other operand is fetched in exactly that row order ("CPERM order") with two transposing LDS reads.
+#pragma once
+
+#include "common.hpp"
+
+namespace segpt {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kBK = 64;        // streamed rows per LDS tile
+constexpr int kThreadsM = 256; // 4 waves
+
+template <int D>
+struct Tile {
+  static constexpr int kRS = D + 8;                 // LDS row stride in bf16 elements (16 B pad)
+  static constexpr int kElems = kBK * kRS;          // elements of one staged tile
+  static constexpr int kTPR = D / 8;                // threads per row when staging (16 B each)
+  static constexpr int kRowsPerPass = kThreadsM / kTPR;
+  static constexpr int kPasses = kBK / kRowsPerPass;  // 16-byte loads per thread per tile
+};
+
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// value held by lane l^32 combined with the own value
+__device__ __forceinline__ float half_max(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_sum(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// sum over the kTPR adjacent lanes that stage one row
+template <int TPR>
+__device__ __forceinline__ float row_group_sum(float x) {
+#pragma unroll
+  for (int o = 1; o < TPR; o <<= 1) x += __shfl_xor(x, o, 64);
+  return x;
+}
+
+__device__ __forceinline__ float sumsq8(u32x4 v) {
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float lo = bf16lo(v[i]), hi = bf16hi(v[i]);
+    s += lo * lo + hi * hi;
+  }
+  return s;
+}
+__device__ __forceinline__ u32x4 scale8(u32x4 v, float f) {
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = pack_bf16x2(bf16lo(v[i]) * f, bf16hi(v[i]) * f);
+  return r;
+}
+__device__ __forceinline__ u32x4 mix8(u32x4 a, u32x4 b, float ca, float cb) {
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    r[i] = pack_bf16x2(ca * bf16lo(a[i]) + cb * bf16lo(b[i]), ca * bf16hi(a[i]) + cb * bf16hi(b[i]));
+  return r;
+}
+
+// A/B fragment of a row-major LDS tile for the 32-row block `rb`, contraction step `ks` (16 columns):
+// lane reads 16 contiguous bytes at row 32*rb + l%32, column 16*ks + 8*(l/32).
+template <int D>
+__device__ __forceinline__ bf16x8 frag_rowmajor(const uint16_t* tile, int rb, int ks, int lane) {
+  const uint16_t* p = tile + (32 * rb + (lane & 31)) * Tile<D>::kRS + 16 * ks + 8 * (lane >> 5);
+  return as_bf16x8(*reinterpret_cast<const u32x4*>(p));
+}
+
+// Transposed fragment of a row-major LDS tile [row][col]: the lane's MFMA row is a COLUMN of the tile
+// (col = 32*cb + l%32) and its 8 contraction entries are tile rows in CPERM order
+//   16*s + {4hh..4hh+3, 8+4hh..8+4hh+3}.
+// ds_read_b64_tr_b16 semantics (per 16-lane group, source lane r gives the address of 4 elements):
+//   result[lane i][e] = LDS[addr(4e + i/4) + i%4]
+// so source lane r points at row base + r/4, column cbase + 4*(r%4) and lane i receives column cbase + i,
+// rows base..base+3.
+template <int D>
+__device__ __forceinline__ bf16x8 frag_transposed(const uint16_t* tile, int cb, int s, int lane) {
+  const int r = lane & 15;
+  const int hh = lane >> 5;
+  const int col = 32 * cb + 16 * ((lane >> 4) & 1) + 4 * (r & 3);
+  const int row = 16 * s + 4 * hh + (r >> 2);
+  const uint16_t* p = tile + row * Tile<D>::kRS + col;
+  typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 8 * Tile<D>::kRS));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+// pack registers 8s..8s+7 of a C tile into a bf16 operand (CPERM order)
+__device__ __forceinline__ bf16x8 pack_c_half(const f32x16& c, int s) {
+  u32x4 w;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(c[8 * s + 2 * i], c[8 * s + 2 * i + 1]);
+  return as_bf16x8(w);
+}
+
+// ---- K/V tile staging: global -> registers (16 B per thread per pass) -> normalise / mix -> LDS (row-major)
+template <int D>
+struct StageRegs {
+  u32x4 k[Tile<D>::kPasses], v[Tile<D>::kPasses], vf[Tile<D>::kPasses];
+};
+
+template <int D, bool VR>
+__device__ __forceinline__ void stage_load(const segpt_attn_params& p, int b, int g, int j0, StageRegs<D>& r) {
+  using T = Tile<D>;
+  const int tid = threadIdx.x;
+  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
+#pragma unroll
+  for (int ps = 0; ps < T::kPasses; ++ps) {
+    const int j = j0 + r0 + ps * T::kRowsPerPass;
+    if (j < p.Sk) {
+      r.k[ps] = *reinterpret_cast<const u32x4*>(row_ptr<uint16_t>(p.k, b, g, j) + chunk * 8);
+      r.v[ps] = *reinterpret_cast<const u32x4*>(row_ptr<uint16_t>(p.v, b, g, j) + chunk * 8);
+      if (VR) r.vf[ps] = *reinterpret_cast<const u32x4*>(row_ptr<uint16_t>(p.v_first, b, g, j) + chunk * 8);
+    } else {
+      r.k[ps] = u32x4{0, 0, 0, 0};
+      r.v[ps] = u32x4{0, 0, 0, 0};
+      if (VR) r.vf[ps] = u32x4{0, 0, 0, 0};
+    }
+  }
+}
+
+template <int D, bool VR>
+__device__ __forceinline__ void stage_store(const StageRegs<D>& r, uint16_t* kt, uint16_t* vt, float eps, float c1, float c2) {
+  using T = Tile<D>;
+  const int tid = threadIdx.x;
+  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
+#pragma unroll
+  for (int ps = 0; ps < T::kPasses; ++ps) {
+    const int row = r0 + ps * T::kRowsPerPass;
+    const float ss = row_group_sum<T::kTPR>(sumsq8(r.k[ps]));
+    const float beta = fast_rsq(ss * (1.0f / D) + eps);
+    *reinterpret_cast<u32x4*>(kt + row * T::kRS + chunk * 8) = scale8(r.k[ps], beta);
+    *reinterpret_cast<u32x4*>(vt + row * T::kRS + chunk * 8) = VR ? mix8(r.v[ps], r.vf[ps], c1, c2) : r.v[ps];
+  }
+}
+
+// Decode a 1-D workgroup id into (tile, head, batch).  Heavy (late) tiles are issued first and,
+// when the number of (batch, kv head) pairs is a multiple of 8, every pair is pinned to one XCD
+// (workgroups are dealt round-robin over the 8 XCDs) so that all query heads of a GQA group and all
+// their tiles read K/V through the same L2.
+struct WgCoord {
+  int tile, b, g, hh;
+};
+__device__ __forceinline__ WgCoord decode_wg(int bid, int n_tiles, int B, int Hkv, int rep) {
+  const int pairs = B * Hkv;
+  int xcd = 0, slot = bid, pp = pairs;
+  if ((pairs & 7) == 0) {
+    xcd = bid & 7;
+    slot = bid >> 3;
+    pp = pairs >> 3;
+  }
+  const int per_tile = pp * rep;
+  const int trev = slot / per_tile;
+  const int rem = slot - trev * per_tile;
+  const int pl = rem / rep;
+  WgCoord c;
+  c.hh = rem - pl * rep;
+  const int pair = ((pairs & 7) == 0) ? pl * 8 + xcd : pl;
+  c.b = pair / Hkv;
+  c.g = pair - c.b * Hkv;
+  c.tile = n_tiles - 1 - trev;
+  return c;
+}
+
+}  // namespace segpt

@@ -1,0 +1,143 @@
+// HBM-bound helper kernels of the backward:
+//   bwd_pre     delta_i = rowsum(dY_i * Y_i); with a gate also dgate = (1 - sigmoid(z)) * delta and
+//               dO_eff = gate_scale * sigmoid(z) * dY  (Y is the saved, already gated output, so
+//               rowsum(dO_eff * O) == rowsum(dY * Y) and no division by the gate is needed).
+//   bwd_reduce  second stage of the scale-gradient reduction: sums the per-workgroup partial
+//               vectors and applies dg_q = g_k * dg, dg_k = g_q * dg (the logits depend on the two
+//               scale vectors only through their product); also sums the (dc1, dc2) partials.
+#include "common.hpp"
+
+namespace segpt {
+namespace {
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void bwd_pre_kernel(KArgs a) {
+  const segpt_attn_params& p = a.p;
+  constexpr int V = Elem<T>::kVec;
+  constexpr int TPR = D / V;          // threads per row
+  constexpr int RPB = 256 / TPR;      // rows per block
+  const int tid = threadIdx.x;
+  const int part = tid % TPR;
+  const int64_t rid = (int64_t)blockIdx.x * RPB + tid / TPR;  // flat (b, h, s)
+  const int64_t nrows = (int64_t)p.B * p.H * p.Sq;
+  const bool live = rid < nrows;
+  const int64_t r = live ? rid : nrows - 1;
+  const int s = (int)(r % p.Sq);
+  const int h = (int)((r / p.Sq) % p.H);
+  const int b = (int)(r / ((int64_t)p.Sq * p.H));
+  float y[V], dy[V];
+  Elem<T>::load(row_ptr<T>(p.o, b, h, s) + part * V, y);
+  Elem<T>::load(row_ptr<T>(p.d_o, b, h, s) + part * V, dy);
+  float acc = 0.f;
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc += y[e] * dy[e];
+#pragma unroll
+  for (int o = 1; o < TPR; o <<= 1) acc += __shfl_xor(acc, o, 64);
+  if (!live) return;
+  if (part == 0) a.delta[r] = acc;
+  if (p.gate.ptr) {
+    const int64_t gi = (int64_t)b * p.gate.stride_b + (int64_t)s * p.gate.stride_s + (int64_t)h * p.gate.stride_h;
+    const float z = Elem<T>::load1(reinterpret_cast<const T*>(p.gate.ptr) + gi);
+    const float sg = sigmoidf_acc(z);
+    if (part == 0) {
+      const int64_t di = (int64_t)b * p.dgate.stride_b + (int64_t)s * p.dgate.stride_s + (int64_t)h * p.dgate.stride_h;
+      Elem<T>::store1(reinterpret_cast<T*>(p.dgate.ptr) + di, (1.0f - sg) * acc);
+    }
+    const float f = p.gate_scale * sg;
+#pragma unroll
+    for (int e = 0; e < V; ++e) dy[e] *= f;
+    Elem<T>::store(reinterpret_cast<T*>(a.do_eff) + r * D + part * V, dy);
+  }
+}
+
+__global__ __launch_bounds__(256) void bwd_reduce_kernel(KArgs a) {
+  const segpt_attn_params& p = a.p;
+  __shared__ float red[256];
+  __shared__ float tot[128];
+  const int tid = threadIdx.x;
+  const int D = p.D;
+  const int lanes = 256 / D;  // threads cooperating on one d (2, 4 or 8)
+  const int d = tid % D, sl = tid / D;
+  float acc = 0.f;
+  for (int blk = sl; blk < a.n_dq_blocks; blk += lanes) acc += a.dg_part[(int64_t)blk * D + d];
+  red[tid] = acc;
+  __syncthreads();
+  if (tid < D) {
+    float t = 0.f;
+    for (int x = 0; x < lanes; ++x) t += red[x * D + tid];
+    tot[tid] = t;
+  }
+  __syncthreads();
+  if (tid < D) {
+    if (p.gq_numel == D) {
+      const float gk = p.gk_numel == 0 ? 1.f : (p.gk_numel == 1 ? p.g_k[0] : p.g_k[tid]);
+      p.dg_q[tid] = gk * tot[tid];
+    }
+    if (p.gk_numel == D) {
+      const float gq = p.gq_numel == 1 ? p.g_q[0] : p.g_q[tid];
+      p.dg_k[tid] = gq * tot[tid];
+    }
+  }
+  if (tid == 0) {
+    if (p.gq_numel == 1) {
+      float t = 0.f;
+      for (int x = 0; x < D; ++x) {
+        const float gk = p.gk_numel == 0 ? 1.f : (p.gk_numel == 1 ? p.g_k[0] : p.g_k[x]);
+        t += gk * tot[x];
+      }
+      p.dg_q[0] = t;
+    }
+    if (p.gk_numel == 1) {
+      float t = 0.f;
+      for (int x = 0; x < D; ++x) {
+        const float gq = p.gq_numel == 1 ? p.g_q[0] : p.g_q[x];
+        t += gq * tot[x];
+      }
+      p.dg_k[0] = t;
+    }
+  }
+  if (p.vr_coef) {
+    __syncthreads();
+    float s1 = 0.f, s2 = 0.f;
+    for (int blk = tid; blk < a.n_dkdv_blocks; blk += 256) {
+      s1 += a.dcoef_part[(int64_t)blk * 2];
+      s2 += a.dcoef_part[(int64_t)blk * 2 + 1];
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) { s1 += __shfl_xor(s1, o, 64); s2 += __shfl_xor(s2, o, 64); }
+    if ((tid & 63) == 0) { red[(tid >> 6) * 2] = s1; red[(tid >> 6) * 2 + 1] = s2; }
+    __syncthreads();
+    if (tid < 2) p.dvr_coef[tid] = red[tid] + red[2 + tid] + red[4 + tid] + red[6 + tid];
+  }
+}
+
+template <typename T>
+int launch_pre_t(const KArgs& a, hipStream_t st) {
+  const segpt_attn_params& p = a.p;
+  const int64_t nrows = (int64_t)p.B * p.H * p.Sq;
+  constexpr int V = Elem<T>::kVec;
+  const int rpb = 256 / (p.D / V);
+  dim3 grid((unsigned)((nrows + rpb - 1) / rpb)), block(256);
+  switch (p.D) {
+    case 32:
+      if constexpr (sizeof(T) == 4) { hipLaunchKernelGGL((bwd_pre_kernel<T, 32>), grid, block, 0, st, a); break; }
+      return (int)hipErrorInvalidValue;
+    case 64: hipLaunchKernelGGL((bwd_pre_kernel<T, 64>), grid, block, 0, st, a); break;
+    case 128: hipLaunchKernelGGL((bwd_pre_kernel<T, 128>), grid, block, 0, st, a); break;
+    default: return (int)hipErrorInvalidValue;
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace
+
+int launch_bwd_pre(const KArgs& a, hipStream_t st) {
+  return a.p.dtype == SEGPT_DTYPE_FP32 ? launch_pre_t<float>(a, st) : launch_pre_t<uint16_t>(a, st);
+}
+
+int launch_bwd_reduce(const KArgs& a, hipStream_t st) {
+  hipLaunchKernelGGL(bwd_reduce_kernel, dim3(1), dim3(256), 0, st, a);
+  return (int)hipGetLastError();
+}
+
+}  // namespace segpt

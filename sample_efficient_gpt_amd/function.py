@@ -1,0 +1,247 @@
+"""Autograd front end of the fused QK-norm flash attention (HIP kernels behind a C ABI).
+
+Two entry points share one implementation:
+
+* ``QKNormFlashAttnFunc.apply(Q, K, V, gain, is_causal=True, q_start=0, ...)`` -- positional drop-in
+  for the reference's ``TritonFlashAttnQKNormFunc``
+  (sample_efficient_gpt/transformer/ops/triton_flash_attn_qknorm.py:262-343): flattened
+  ``[(h b), S, d]`` tensors, gradients for ``Q, K, V, gain`` and ``None`` for the flags.  Optional
+  trailing positionals switch on what the reference's caller does around the op
+  (sample_efficient_gpt/transformer/attention.py:207-255): un-expanded GQA K/V, the value-residual
+  mix, the per-head sigmoid gate, a k-side scale vector.
+* ``qknorm_attention(q, k, v, g_q, ...)`` -- the same op on canonical ``[B, H, S, D]`` /
+  ``[B, Hkv, S, D]`` views with keyword arguments.
+
+Defaults follow the live module (attention.py:51-80): RMS normaliser, eps 1e-6 on the mean,
+logits scaled by 1/sqrt(d).  ``eps=1e-8/d, sm_scale=1/d`` reproduces the fused Triton kernel's
+own formula (triton_flash_attn_qknorm.py:67-91).
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.bfloat16: _lib.SEGPT_DTYPE_BF16, torch.float32: _lib.SEGPT_DTYPE_FP32}
+
+
+def _scale_arg(g, device):
+    """Scale parameter -> contiguous fp32 device vector (or None)."""
+    if g is None:
+        return None
+    return g.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+
+
+def _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start):
+    B, H, Sq, D = q.shape
+    p.dtype = _DTYPES[q.dtype]
+    p.B, p.H, p.Hkv, p.Sq, p.Sk, p.D = B, H, k.shape[1], Sq, k.shape[2], D
+    p.causal = int(bool(causal))
+    p.q_start = int(q_start)
+    p.gq_numel = g_q.numel()
+    p.gk_numel = 0 if g_k is None else g_k.numel()
+    p.eps, p.sm_scale, p.gate_scale = float(eps), float(sm_scale), float(gate_scale)
+    p.q, p.k, p.v, p.o = _lib.t4(q), _lib.t4(k), _lib.t4(v), _lib.t4(y)
+    p.v_first = _lib.t4(v_first)
+    p.gate = _lib.t3(gate)
+    p.lse = _lib.ptr(lse)
+    p.g_q, p.g_k, p.vr_coef = _lib.ptr(g_q), _lib.ptr(g_k), _lib.ptr(vr_coef)
+
+
+def _check_inputs(q, k, v, g_q, g_k, v_first, vr_coef, gate):
+    if q.dtype not in _DTYPES:
+        raise TypeError(f"qknorm attention supports bfloat16 and float32 tensors, got {q.dtype}")
+    for name, t in (("k", k), ("v", v), ("v_first", v_first), ("gate_logits", gate)):
+        if t is not None and t.dtype != q.dtype:
+            raise TypeError(f"{name} has dtype {t.dtype}, expected {q.dtype}")
+    assert q.is_cuda and k.is_cuda and v.is_cuda, "q, k, v must be device tensors"
+    B, H, Sq, D = q.shape
+    assert k.dim() == 4 and v.shape == k.shape and k.shape[0] == B and k.shape[3] == D, "k/v shape mismatch"
+    assert H % k.shape[1] == 0, "number of query heads must be a multiple of the kv heads"
+    assert g_q.numel() in (1, D), "gain must have 1 or head_dim elements"
+    assert g_k is None or g_k.numel() in (1, D), "k_gain must have 1 or head_dim elements"
+    assert (v_first is None) == (vr_coef is None), "v_first and vr_coef go together"
+    if v_first is not None:
+        assert v_first.shape == v.shape and vr_coef.numel() == 2
+    if gate is not None:
+        assert gate.shape == (B, Sq, H), "gate_logits must be [B, Sq, H]"
+
+
+def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y):
+    """Launch the forward on canonical 4-D views; returns lse [B,H,Sq] fp32.  `y` is written."""
+    lib = _lib.load()
+    B, H, Sq, _ = q.shape
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    p = _lib.new_params()
+    _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start)
+    rc = lib.segpt_attn_fwd(p, torch.cuda.current_stream(q.device).cuda_stream)
+    if rc != 0:
+        raise _lib.SegptError(rc, "segpt_attn_fwd")
+    return lse
+
+
+def _backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y, lse, dy,
+              dq, dk, dv, dv_first, dgate):
+    """Launch the backward; dq/dk/dv(/dv_first/dgate) are written; returns (dg_q, dg_k, dvr_coef) fp32."""
+    lib = _lib.load()
+    dev = q.device
+    dg_q = torch.empty_like(g_q)
+    dg_k = None if g_k is None else torch.empty_like(g_k)
+    dcoef = None if vr_coef is None else torch.empty(2, dtype=torch.float32, device=dev)
+    p = _lib.new_params()
+    _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start)
+    p.d_o, p.dq, p.dk, p.dv = _lib.t4(dy), _lib.t4(dq), _lib.t4(dk), _lib.t4(dv)
+    p.dv_first = _lib.t4(dv_first)
+    p.dgate = _lib.t3(dgate)
+    p.dg_q, p.dg_k, p.dvr_coef = _lib.ptr(dg_q), _lib.ptr(dg_k), _lib.ptr(dcoef)
+    nbytes = lib.segpt_attn_workspace_bytes(p, 1)
+    ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=dev)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    rc = lib.segpt_attn_bwd(p, torch.cuda.current_stream(dev).cuda_stream)
+    if rc != 0:
+        raise _lib.SegptError(rc, "segpt_attn_bwd")
+    return dg_q, dg_k, dcoef
+
+
+def _lastdim_contig(x):
+    return x if x.stride(-1) == 1 else x.contiguous()
+
+
+class _CoreFunc(torch.autograd.Function):
+    """Canonical-layout op: q [B,H,Sq,D], k/v/v_first [B,Hkv,Sk,D], gate [B,Sq,H]."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start):
+        gq32, gk32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device)
+        coef32 = None if vr_coef is None else vr_coef.detach().to(device=q.device, dtype=torch.float32).reshape(-1).contiguous()
+        _check_inputs(q, k, v, gq32, gk32, v_first, coef32, gate)
+        q, k, v = _lastdim_contig(q), _lastdim_contig(k), _lastdim_contig(v)
+        v_first = None if v_first is None else _lastdim_contig(v_first)
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(q.shape[-1])
+        y = torch.empty_like(q)
+        if y.stride(-1) != 1:
+            y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        lse = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y)
+        ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse)
+        ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start)
+        ctx.mark_non_differentiable(lse)
+        return y, lse
+
+    @staticmethod
+    def backward(ctx, dy, _dlse):
+        q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse = ctx.saved_tensors
+        gate_scale, eps, sm_scale, causal, q_start = ctx.cfg
+        gq32, gk32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device)
+        coef32 = None if vr_coef is None else vr_coef.detach().to(device=q.device, dtype=torch.float32).reshape(-1).contiguous()
+        dy = _lastdim_contig(dy)
+        if dy.dtype != q.dtype:
+            dy = dy.to(q.dtype)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dv_first = None if v_first is None else torch.empty_like(v_first)
+        dgate = None if gate is None else torch.empty_like(gate)
+        dg_q, dg_k, dcoef = _backward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal,
+                                      q_start, y, lse, dy, dq, dk, dv, dv_first, dgate)
+        dg_q = dg_q.reshape(g_q.shape).to(g_q.dtype)
+        if g_k is not None:
+            dg_k = dg_k.reshape(g_k.shape).to(g_k.dtype)
+        if vr_coef is not None:
+            dcoef = dcoef.reshape(vr_coef.shape).to(vr_coef.dtype)
+        return dq, dk, dv, dg_q, dg_k, dv_first, dcoef, dgate, None, None, None, None, None
+
+
+def qknorm_attention(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate_logits=None, gate_scale=2.0,
+                     eps=1e-6, sm_scale=None, causal=True, q_start=0, return_lse=False):
+    """Fused QK-norm attention on canonical views.
+
+    q ``[B,H,Sq,D]``; k, v, v_first ``[B,Hkv,Sk,D]`` (any strides, last dim contiguous, rows 16 B
+    aligned); g_q, g_k scale parameters of 1 or D elements; vr_coef device tensor ``[2]`` = (c1, c2)
+    with ``v' = c1 v + c2 v_first``; gate_logits ``[B,Sq,H]`` with ``y = gate_scale*sigmoid(z)*o``.
+    """
+    y, lse = _CoreFunc.apply(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start)
+    return (y, lse) if return_lse else y
+
+
+def _canon(x, n_heads):
+    """[(h b), S, d] -> [B, H, S, d] view (no copy): head-major flatten of attention.py:199."""
+    n, S, d = x.shape
+    return x.view(n_heads, n // n_heads, S, d).permute(1, 0, 2, 3)
+
+
+class QKNormFlashAttnFunc(torch.autograd.Function):
+    """Drop-in for ``TritonFlashAttnQKNormFunc`` (triton_flash_attn_qknorm.py:262-343).
+
+    ``apply(Q, K, V, gain, is_causal=True, q_start=0, k_gain=None, v_first=None, vr_coef=None,
+    gate_logits=None, gate_scale=2.0, n_kv_heads=None, eps=1e-6, sm_scale=None)`` -- positional only,
+    as autograd Functions are.  ``Q [(h b), Nq, d]``, ``K, V [(h b) or (hkv b), Nk, d]`` contiguous
+    device tensors (2-D inputs are promoted to 3-D, the output stays 3-D, :278-281).  When K/V carry
+    fewer rows than Q they are un-expanded GQA tensors and ``n_kv_heads`` is required; query row
+    ``n = h*B + b`` then reads kv row ``(h // rep)*B + b`` exactly as the reference's
+    ``repeat_interleave`` expansion does (attention.py:207-218).  Returns ``O`` with Q's shape and dtype.
+    """
+
+    @staticmethod
+    def forward(ctx, Q, K, V, gain, is_causal=True, q_start=0, k_gain=None, v_first=None, vr_coef=None,
+                gate_logits=None, gate_scale=2.0, n_kv_heads=None, eps=1e-6, sm_scale=None):
+        assert Q.is_cuda and Q.is_contiguous()
+        assert K.is_cuda and K.is_contiguous()
+        assert V.is_cuda and V.is_contiguous()
+        assert gain.is_cuda
+        if Q.ndim == 2:
+            Q, K, V = Q.unsqueeze(0), K.unsqueeze(0), V.unsqueeze(0)
+            if v_first is not None and v_first.ndim == 2:
+                v_first = v_first.unsqueeze(0)
+        nq, nk = Q.shape[0], K.shape[0]
+        if nk != nq or n_kv_heads is not None or gate_logits is not None:
+            if n_kv_heads is None:
+                assert gate_logits is not None and nk == nq, "n_kv_heads is required for un-expanded GQA K/V"
+                H = Hkv = gate_logits.shape[-1]
+            else:
+                Hkv = int(n_kv_heads)
+                assert nq % nk == 0 and nk % Hkv == 0, "K/V rows must be n_kv_heads * batch"
+                H = Hkv * (nq // nk)
+        else:
+            H = Hkv = 1  # every flattened row is its own (batch, head): plain MHA layout of the reference
+        if v_first is not None:
+            assert v_first.is_cuda and v_first.is_contiguous()
+        q4, k4, v4 = _canon(Q, H), _canon(K, Hkv), _canon(V, Hkv)
+        vf4 = None if v_first is None else _canon(v_first, Hkv)
+        gq32, gk32 = _scale_arg(gain, Q.device), _scale_arg(k_gain, Q.device)
+        coef32 = None if vr_coef is None else vr_coef.detach().to(device=Q.device, dtype=torch.float32).reshape(-1).contiguous()
+        _check_inputs(q4, k4, v4, gq32, gk32, vf4, coef32, gate_logits)
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(Q.shape[-1])
+        O = torch.empty_like(Q)
+        lse = _forward(q4, k4, v4, gq32, gk32, vf4, coef32, gate_logits, gate_scale, eps, sm_scale, is_causal, q_start,
+                       _canon(O, H))
+        ctx.save_for_backward(lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate_logits)
+        ctx.cfg = (H, Hkv, gate_scale, eps, sm_scale, bool(is_causal), int(q_start))
+        return O
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate = ctx.saved_tensors
+        H, Hkv, gate_scale, eps, sm_scale, causal, q_start = ctx.cfg
+        grad_output = grad_output.contiguous()
+        if grad_output.dtype != Q.dtype:
+            grad_output = grad_output.to(Q.dtype)
+        if grad_output.ndim == 2:
+            grad_output = grad_output.unsqueeze(0)
+        dQ, dK, dV = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+        dVf = None if v_first is None else torch.empty_like(v_first)
+        dgate = None if gate is None else torch.empty_like(gate)
+        gq32, gk32 = _scale_arg(gain, Q.device), _scale_arg(k_gain, Q.device)
+        coef32 = None if vr_coef is None else vr_coef.detach().to(device=Q.device, dtype=torch.float32).reshape(-1).contiguous()
+        dg_q, dg_k, dcoef = _backward(
+            _canon(Q, H), _canon(K, Hkv), _canon(V, Hkv), gq32, gk32,
+            None if v_first is None else _canon(v_first, Hkv), coef32, gate, gate_scale, eps, sm_scale, causal, q_start,
+            _canon(O, H), lse, _canon(grad_output, H), _canon(dQ, H), _canon(dK, Hkv), _canon(dV, Hkv),
+            None if dVf is None else _canon(dVf, Hkv), dgate)
+        dgain = dg_q.reshape(gain.shape).to(gain.dtype)
+        dk_gain = None if k_gain is None else dg_k.reshape(k_gain.shape).to(k_gain.dtype)
+        dcoef = None if vr_coef is None else dcoef.reshape(vr_coef.shape).to(vr_coef.dtype)
+        #      Q   K   V   gain   causal q_start k_gain  v_first vr_coef gate  gate_scale n_kv eps sm_scale
+        return dQ, dK, dV, dgain, None, None, dk_gain, dVf, dcoef, dgate, None, None, None, None

@@ -1,0 +1,104 @@
+"""Shared helpers for the GPU parity tests: run the HIP op, run the CPU oracle, compare."""
+
+from __future__ import annotations
+
+import torch
+
+from oracle import qknorm_attn_oracle as orc
+from sample_efficient_gpt_amd import qknorm_attention
+
+# north-star tolerances: bf16 kernels vs an fp32/fp64 reference: 2e-2 max-abs / 1e-2 relative; fp32 path: 1e-5
+TOL = {torch.bfloat16: dict(atol=2e-2, rtol=1e-2), torch.float32: dict(atol=1e-5, rtol=1e-5)}
+
+
+def gen(B, H, Hkv, Sq, Sk, D, dtype, *, extras=False, scalar_gain=False, no_gk=False, seed=0, head_scales=False):
+    g = torch.Generator().manual_seed(seed)
+
+    def n(*s):
+        return torch.randn(*s, generator=g, dtype=torch.float32)
+
+    x = {"q": n(B, H, Sq, D), "k": n(B, Hkv, Sk, D), "v": n(B, Hkv, Sk, D), "d_o": n(B, H, Sq, D)}
+    if head_scales:
+        x["q"] *= 0.5 + 1.5 * torch.rand(1, H, 1, 1, generator=g)
+        x["k"] *= 0.5 + 1.5 * torch.rand(1, Hkv, 1, 1, generator=g)
+        x["v"] *= 0.5 + 1.5 * torch.rand(1, Hkv, 1, 1, generator=g)
+    x = {k: t.to(dtype) for k, t in x.items()}
+    x["g_q"] = torch.tensor([1.3]) if scalar_gain else 1.0 + 0.02 * n(D)
+    x["g_k"] = None if no_gk else 1.0 + 0.02 * n(D)
+    if extras:
+        x["gate_logits"] = n(B, Sq, H).to(dtype)
+        x["v_first"] = n(B, Hkv, Sk, D).to(dtype)
+        lam = 0.3 + 0.4 * torch.rand(1, generator=g)
+        x["vr_coef"] = torch.cat([lam, 1 - lam])
+    return x
+
+
+def run_gpu(x, device, *, backward=True, **kw):
+    """Run the HIP op (and its backward) on `device`; returns CPU tensors."""
+    names = ["q", "k", "v", "g_q", "g_k", "v_first", "vr_coef", "gate_logits"]
+    t = {n: (x[n].to(device).requires_grad_(backward) if x.get(n) is not None else None) for n in names}
+    y, lse = qknorm_attention(t["q"], t["k"], t["v"], t["g_q"], t["g_k"], v_first=t["v_first"], vr_coef=t["vr_coef"],
+                              gate_logits=t["gate_logits"], return_lse=True, **kw)
+    out = {"y": y.detach().cpu(), "lse": lse.detach().cpu()}
+    if backward:
+        y.backward(x["d_o"].to(device))
+        for n, gname in (("q", "dq"), ("k", "dk"), ("v", "dv"), ("g_q", "dg_q"), ("g_k", "dg_k"), ("v_first", "dv_first"),
+                         ("vr_coef", "dvr_coef"), ("gate_logits", "dgate_logits")):
+            if t[n] is not None:
+                out[gname] = t[n].grad.detach().cpu()
+    torch.cuda.synchronize()
+    return out
+
+
+def run_oracle(x, *, backward=True, odtype=torch.float64, **kw):
+    """CPU oracle on the same bits, computed in `odtype`."""
+    f = lambda n: None if x.get(n) is None else x[n].to(odtype)
+    okw = dict(kw)
+    if f("v_first") is not None:
+        okw.update(v_first=f("v_first"), vr_coef=f("vr_coef"))
+    if f("gate_logits") is not None:
+        okw.update(gate_logits=f("gate_logits"))
+    if not backward:
+        y, lse, _, _ = orc.attention_forward(f("q"), f("k"), f("v"), f("g_q"), f("g_k"), **okw)
+        return {"y": y, "lse": lse}
+    return orc.attention_backward_autograd(f("q"), f("k"), f("v"), f("g_q"), f("g_k"), f("d_o"), **okw)
+
+
+# Parameter gradients that are sums over every (batch, head, row): each summand carries its own bf16
+# rounding noise, so the error of the sum scales with the norm of the summands, not with the (possibly
+# cancelling) value of one entry.  For these the relative part of the tolerance is taken against the
+# largest entry of the reference vector (norm-wise), everything else is compared element-wise.
+REDUCED = ("dg_q", "dg_k", "dg", "dvr_coef")
+
+
+def scalar_gain_scale(x, **kw):
+    """Yardstick for the gradient of a SCALAR gain: it is the sum over d of the per-dimension scale
+    gradients, whose rounding errors add up, so the relative tolerance is taken against
+    sum_d |dg_d| of the oracle's vector-mode gradient rather than against the cancelled total."""
+    D = x["q"].shape[-1]
+    xv = dict(x)
+    xv["g_q"] = x["g_q"].reshape(-1).expand(D).clone()
+    ref = run_oracle(xv, **kw)
+    return {"dg_q": float(ref["dg_q"].abs().sum())}
+
+
+def compare(got, ref, dtype, names=None, label="", scales=None):
+    """Asserts |got - ref| <= atol + rtol*|ref| for every output; returns {name: max_abs_err}.
+    `scales` overrides the magnitude the relative part refers to for the named outputs."""
+    tol = TOL[dtype]
+    errs = {}
+    for n in (names or ref.keys()):
+        r = ref[n].double()
+        g = got[n].double().reshape(r.shape)
+        assert torch.isfinite(g).all(), f"{label}{n}: non-finite values"
+        err = (g - r).abs()
+        scale = r.abs().max() if n in REDUCED else r.abs()
+        if scales and n in scales:
+            scale = max(float(r.abs().max()), scales[n])
+        bound = tol["atol"] + tol["rtol"] * scale
+        errs[n] = float(err.max())
+        bad = err > bound
+        assert not bad.any(), (
+            f"{label}{n}: {int(bad.sum())}/{bad.numel()} outside tolerance, max abs err {errs[n]:.3e} "
+            f"(ref max {float(r.abs().max()):.3e})")
+    return errs

@@ -1,0 +1,180 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads, exports what the header declares,
+validates arguments before any launch, and the Python front end keeps the reference's signature."""
+
+import ctypes as C
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+from sample_efficient_gpt_amd import QKNormFlashAttnFunc, SelfDotProductAttnQKNorm, TritonFlashAttnQKNormFunc, _lib
+from sample_efficient_gpt_amd import CONFIGS, make_inputs
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "segpt_attn.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"^\s*(?:const\s+)?[A-Za-z_][\w\s\*]*?\b(segpt_\w+)\s*\(", text, flags=re.M)
+
+
+def test_library_exports_every_declared_symbol(lib):
+    declared = _declared_functions()
+    assert set(declared) == set(_lib.EXPORTED_SYMBOLS), declared
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.segpt_abi_version() == _lib.SEGPT_ABI_VERSION
+
+
+def test_header_constants_match_binding():
+    text = open(HEADER).read()
+    consts = dict(re.findall(r"#define\s+(SEGPT_\w+)\s+(-?\d+)", text))
+    assert int(consts["SEGPT_ABI_VERSION"]) == _lib.SEGPT_ABI_VERSION
+    assert int(consts["SEGPT_DTYPE_BF16"]) == _lib.SEGPT_DTYPE_BF16
+    assert int(consts["SEGPT_DTYPE_FP32"]) == _lib.SEGPT_DTYPE_FP32
+    # every error code has its own text
+    texts = {_lib.strerror(int(v)) for k, v in consts.items() if k.startswith("SEGPT_E_")}
+    assert len(texts) == len([k for k in consts if k.startswith("SEGPT_E_")])
+    assert _lib.strerror(0) == "ok" and "HIP" in _lib.strerror(700)
+
+
+def _valid_params(dtype=_lib.SEGPT_DTYPE_BF16, D=64):
+    """Params with plausible (fake, never dereferenced) device addresses: validation happens on the host."""
+    p = _lib.new_params()
+    p.dtype = dtype
+    p.B, p.H, p.Hkv, p.Sq, p.Sk, p.D = 2, 6, 2, 128, 128, D
+    p.causal, p.q_start, p.gq_numel, p.gk_numel = 1, 0, D, 0
+    p.eps, p.sm_scale, p.gate_scale = 1e-6, 0.125, 2.0
+    fake = 0x10000
+    for name in ("q", "o", "d_o", "dq"):
+        setattr(p, name, _lib.Tensor4(fake, 6 * 128 * D, 128 * D, D))
+    for name in ("k", "v", "dk", "dv"):
+        setattr(p, name, _lib.Tensor4(fake, 2 * 128 * D, 128 * D, D))
+    p.lse = p.g_q = p.dg_q = fake
+    return p
+
+
+def test_argument_errors_are_reported_before_any_launch(lib):
+    # no GPU in this process: every call below must return from host-side validation
+    assert lib.segpt_attn_fwd(None, None) == -1
+    p = _valid_params()
+    p.struct_bytes = 8
+    assert lib.segpt_attn_fwd(p, None) == -2
+    p = _valid_params(); p.dtype = 7
+    assert lib.segpt_attn_fwd(p, None) == -3
+    p = _valid_params(); p.Hkv = 4
+    assert lib.segpt_attn_fwd(p, None) == -4
+    p = _valid_params(); p.Sq = 0
+    assert lib.segpt_attn_fwd(p, None) == -4
+    p = _valid_params(); p.gq_numel = 3
+    assert lib.segpt_attn_fwd(p, None) == -4
+    p = _valid_params(D=48)
+    assert lib.segpt_attn_fwd(p, None) == -5
+    p = _valid_params(dtype=_lib.SEGPT_DTYPE_BF16, D=32)
+    assert lib.segpt_attn_fwd(p, None) == -5
+    p = _valid_params(); p.q.stride_s = 60
+    assert lib.segpt_attn_fwd(p, None) == -6
+    p = _valid_params(); p.k.stride_h = 7
+    assert lib.segpt_attn_fwd(p, None) == -6
+    p = _valid_params(); p.q_start = -1
+    assert lib.segpt_attn_fwd(p, None) == -9
+    p = _valid_params(); p.v.ptr = 0x10004
+    assert lib.segpt_attn_fwd(p, None) == -10
+    p = _valid_params(); p.q.ptr = None
+    assert lib.segpt_attn_fwd(p, None) == -1
+    p = _valid_params(); p.v_first = _lib.Tensor4(0x10000, 2 * 128 * 64, 128 * 64, 64)  # v_first without vr_coef
+    assert lib.segpt_attn_fwd(p, None) == -8
+    # backward-only checks
+    p = _valid_params()
+    assert lib.segpt_attn_bwd(p, None) == -7  # no workspace
+    need = lib.segpt_attn_workspace_bytes(p, 1)
+    p.workspace, p.workspace_bytes = 0x20000, need - 1
+    assert lib.segpt_attn_bwd(p, None) == -7
+    p = _valid_params(); p.dg_q = None
+    assert lib.segpt_attn_bwd(p, None) == -1
+    p = _valid_params(); p.gate = _lib.Tensor3(0x10000, 128 * 6, 6, 1)
+    p.workspace, p.workspace_bytes = 0x20000, 1 << 30
+    assert lib.segpt_attn_bwd(p, None) == -8  # gate without dgate slot
+
+
+def test_workspace_bytes(lib):
+    p = _valid_params()
+    assert lib.segpt_attn_workspace_bytes(p, 0) == 0
+    base = lib.segpt_attn_workspace_bytes(p, 1)
+    rows = 2 * 6 * 128
+    assert base >= rows * 4 and base % 256 == 0
+    p.gate = _lib.Tensor3(0x10000, 128 * 6, 6, 1)
+    assert lib.segpt_attn_workspace_bytes(p, 1) >= base + rows * 64 * 2  # + gated dO copy
+    bad = _valid_params(); bad.struct_bytes = 4
+    assert lib.segpt_attn_workspace_bytes(bad, 1) == 0
+
+
+def test_params_struct_matches_header_field_order():
+    text = open(HEADER).read()
+    body = text[text.index("typedef struct segpt_attn_params {"): text.index("} segpt_attn_params;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        decl = decl.split("{")[-1].strip()
+        if not decl:
+            continue
+        first, *rest = decl.split(",")
+        names.append(re.findall(r"(\w+)\s*$", first.strip())[0])
+        names += [r.strip().lstrip("*") for r in rest]
+    assert names == [f[0] for f in _lib.AttnParams._fields_]
+
+
+def test_function_signature_is_the_reference_one():
+    # reference: forward(ctx, Q, K, V, gain, is_causal=True, q_start=0)  (triton_flash_attn_qknorm.py:264-272)
+    sig = inspect.signature(QKNormFlashAttnFunc.forward)
+    names = list(sig.parameters)
+    assert names[:7] == ["ctx", "Q", "K", "V", "gain", "is_causal", "q_start"]
+    assert sig.parameters["is_causal"].default is True and sig.parameters["q_start"].default == 0
+    for extra in names[7:]:
+        assert sig.parameters[extra].default is not inspect.Parameter.empty  # extras are optional
+    assert TritonFlashAttnQKNormFunc is QKNormFlashAttnFunc
+    assert issubclass(QKNormFlashAttnFunc, torch.autograd.Function)
+
+
+def test_function_asserts_like_the_reference_on_host_tensors():
+    Q = torch.randn(2, 16, 64)
+    with pytest.raises(AssertionError):  # `assert Q.is_cuda and Q.is_contiguous()`, :273
+        QKNormFlashAttnFunc.apply(Q, Q, Q, torch.ones(1))
+
+
+def test_module_interface():
+    m = SelfDotProductAttnQKNorm(64)
+    sd = m.state_dict()
+    assert list(sd) == ["gain"] and sd["gain"].shape == (1,) and sd["gain"].dtype == torch.float32 and float(sd["gain"]) == 1.0
+    sig = inspect.signature(m.forward)
+    assert list(sig.parameters) == ["Q", "K", "V", "is_causal", "q_start"]
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libsegpt_attn.so"))
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.load()
+
+
+def test_input_generators_are_seeded_and_shaped():
+    c = CONFIGS[1]
+    a, b = make_inputs(c), make_inputs(c)
+    assert all(torch.equal(a[k], b[k]) for k in a)
+    assert a["q"].shape == (2, 4, 256, 64) and a["q"].dtype == torch.float32 and a["g_q"].shape == (64,)
+    c4 = CONFIGS[4].scaled(S=64)
+    x = make_inputs(c4)
+    assert x["gate_logits"].shape == (2, 64, 18) and x["v_first"].shape == (2, 6, 64, 64)
+    lam = float(x["vr_coef"][0])
+    assert 0.3 <= lam <= 0.7 and abs(float(x["vr_coef"].sum()) - 1) < 1e-6
+    assert CONFIGS[3].flops() == 7 * 8 * 18 * 2048 * 2048 * 64 and CONFIGS[2].flops() == 2 * 8 * 18 * 2048 * 2048 * 64

@@ -1,0 +1,255 @@
+"""GPU parity: HIP kernels (through the C ABI) vs the CPU oracle on identical seeded inputs.
+
+bf16: |err| <= 2e-2 + 1e-2*|ref| against the fp64 oracle on the same bf16 bits; fp32: 1e-5 (abs and rel).
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import qknorm_attn_oracle as orc
+from sample_efficient_gpt_amd import CONFIGS, QKNormFlashAttnFunc, SelfDotProductAttnQKNorm, make_inputs, qknorm_attention
+from tests.parity_util import compare, gen, run_gpu, run_oracle, scalar_gain_scale
+
+pytestmark = pytest.mark.gpu
+BF16, F32 = torch.bfloat16, torch.float32
+
+
+def _case(device, dtype, B, H, Hkv, Sq, Sk, D, *, backward=True, seed=0, gen_kw=None, **kw):
+    x = gen(B, H, Hkv, Sq, Sk, D, dtype, seed=seed, **(gen_kw or {}))
+    print(f"case dtype={dtype} B={B} H={H} Hkv={Hkv} Sq={Sq} Sk={Sk} D={D} bwd={backward} gen={gen_kw} kw={kw}", flush=True)
+    got = run_gpu(x, device, backward=backward, **kw)
+    ref = run_oracle(x, backward=backward, **kw)
+    scales = None
+    if backward and dtype == BF16 and x["g_q"].numel() == 1:
+        scales = scalar_gain_scale(x, **kw)
+    return compare(got, ref, dtype, scales=scales)
+
+
+# ------------------------------------------------------------------ fp32 path (1e-5)
+
+
+def test_cfg1_fp32_forward(gpu_device):
+    c = CONFIGS[1]
+    x = make_inputs(c)
+    print("cfg1 fp32 forward", flush=True)
+    got = run_gpu(x, gpu_device, backward=False, eps=c.eps, sm_scale=c.sm_scale)
+    ref = run_oracle(x, backward=False, eps=c.eps, sm_scale=c.sm_scale)
+    errs = compare(got, ref, F32)
+    print("cfg1 max abs err", errs)
+
+
+@pytest.mark.parametrize(
+    "B,H,Hkv,Sq,Sk,D,kw,gen_kw",
+    [
+        (2, 4, 4, 256, 256, 64, {}, {}),
+        (1, 6, 2, 100, 100, 64, {}, {"extras": True}),
+        (2, 4, 2, 77, 77, 32, {}, {"scalar_gain": True, "no_gk": True}),
+        (1, 4, 1, 130, 130, 128, {}, {}),
+        (1, 2, 2, 48, 80, 64, {"causal": False}, {}),
+        (1, 3, 3, 40, 104, 64, {"q_start": 64}, {"extras": True}),
+        (1, 2, 1, 64, 64, 64, {"eps": 1e-8 / 64, "sm_scale": 1 / 64}, {"scalar_gain": True, "no_gk": True}),
+        (1, 4, 2, 200, 200, 64, {"gate_scale": 2.0}, {"extras": True, "scalar_gain": True}),  # scalar q gain + vector k scale
+    ],
+)
+def test_fp32_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
+    _case(gpu_device, F32, B, H, Hkv, Sq, Sk, D, gen_kw=gen_kw, **kw)
+
+
+# ------------------------------------------------------------------ bf16 MFMA path
+
+
+@pytest.mark.parametrize(
+    "B,H,Hkv,Sq,Sk,D,kw,gen_kw",
+    [
+        (1, 1, 1, 64, 64, 64, {}, {}),
+        (1, 1, 1, 256, 256, 64, {}, {}),
+        (2, 6, 2, 512, 512, 64, {}, {}),
+        (1, 3, 1, 300, 300, 64, {}, {}),          # ragged: not a multiple of any tile
+        (1, 2, 2, 77, 77, 64, {}, {"scalar_gain": True, "no_gk": True}),
+        (2, 6, 2, 384, 384, 64, {"gate_scale": 1.0}, {"extras": True}),
+        (1, 4, 2, 200, 200, 64, {"gate_scale": 2.0}, {"extras": True, "scalar_gain": True}),
+        (1, 2, 1, 256, 256, 128, {}, {}),
+        (1, 4, 1, 333, 333, 128, {}, {"extras": True, "head_scales": True}),
+        (1, 2, 2, 96, 200, 64, {"causal": False}, {}),
+        (1, 2, 1, 130, 130, 128, {"causal": False}, {}),
+        (1, 3, 3, 72, 200, 64, {"q_start": 128}, {}),
+        (1, 2, 1, 1, 257, 64, {"q_start": 256}, {}),   # decode step: one query against a 257-key cache
+        (8, 2, 1, 128, 128, 64, {}, {}),              # B*Hkv multiple of 8: XCD-pinned workgroup order
+        (1, 2, 2, 128, 128, 64, {"eps": 1e-8 / 64, "sm_scale": 1 / 64}, {"scalar_gain": True, "no_gk": True}),
+    ],
+)
+def test_bf16_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
+    _case(gpu_device, BF16, B, H, Hkv, Sq, Sk, D, gen_kw=gen_kw, **kw)
+
+
+def _slice_check(device, c, pairs, odtype=torch.float64):
+    """Full-size run on the GPU; oracle on single (batch, kv-group) slices (they are independent)."""
+    x = make_inputs(c)
+    kw = dict(eps=c.eps, sm_scale=c.sm_scale)
+    if c.extras:
+        kw["gate_scale"] = c.gate_scale
+    print(f"full-size {c.name}", flush=True)
+    got = run_gpu(x, device, backward=c.backward, **kw)
+    rep = c.H // c.Hkv
+    worst = {}
+    for b, g in pairs:
+        hs = slice(g * rep, (g + 1) * rep)
+        xs = {"q": x["q"][b:b + 1, hs], "k": x["k"][b:b + 1, g:g + 1], "v": x["v"][b:b + 1, g:g + 1],
+              "d_o": x["d_o"][b:b + 1, hs], "g_q": x["g_q"], "g_k": x["g_k"]}
+        if c.extras:
+            xs.update(gate_logits=x["gate_logits"][b:b + 1, :, hs], v_first=x["v_first"][b:b + 1, g:g + 1], vr_coef=x["vr_coef"])
+        ref = run_oracle(xs, backward=c.backward, odtype=odtype, **kw)
+        gs = {"y": got["y"][b:b + 1, hs], "lse": got["lse"][b:b + 1, hs]}
+        names = ["y", "lse"]
+        if c.backward:
+            gs.update(dq=got["dq"][b:b + 1, hs], dk=got["dk"][b:b + 1, g:g + 1], dv=got["dv"][b:b + 1, g:g + 1])
+            names += ["dq", "dk", "dv"]
+            if c.extras:
+                gs.update(dv_first=got["dv_first"][b:b + 1, g:g + 1], dgate_logits=got["dgate_logits"][b:b + 1, :, hs])
+                names += ["dv_first", "dgate_logits"]
+        errs = compare(gs, ref, c.dtype, names=names, label=f"{c.name}[b={b},g={g}] ")
+        for n, e in errs.items():
+            worst[n] = max(worst.get(n, 0.0), e)
+    print(c.name, "worst max-abs errors over slices:", {k: f"{v:.2e}" for k, v in worst.items()}, flush=True)
+    return x, got, kw
+
+
+def test_cfg2_imu1_forward_full_size(gpu_device):
+    _slice_check(gpu_device, CONFIGS[2], [(0, 0), (7, 5), (3, 2)])
+
+
+def test_cfg3_imu1_fwd_bwd_full_size(gpu_device):
+    c = CONFIGS[3]
+    x, got, kw = _slice_check(gpu_device, c, [(0, 0), (7, 5)])
+    # the scale-vector gradients sum over every (b, h, row): check them as a sum of per-batch GPU runs
+    # (additivity), each of which the small cases above compare with the oracle
+    acc_q = torch.zeros(c.D, dtype=torch.float64)
+    acc_k = torch.zeros(c.D, dtype=torch.float64)
+    for b in range(c.B):
+        xb = {n: (t[b:b + 1] if n in ("q", "k", "v", "d_o") else t) for n, t in x.items()}
+        gb = run_gpu(xb, gpu_device, **kw)
+        acc_q += gb["dg_q"].double()
+        acc_k += gb["dg_k"].double()
+    assert torch.allclose(got["dg_q"].double(), acc_q, atol=2e-2, rtol=1e-2)
+    assert torch.allclose(got["dg_k"].double(), acc_k, atol=2e-2, rtol=1e-2)
+    # and one batch of it directly against the oracle
+    xb = {n: (t[:1] if n in ("q", "k", "v", "d_o") else t) for n, t in x.items()}
+    compare(run_gpu(xb, gpu_device, **kw), run_oracle(xb, **kw), c.dtype, names=["dg_q", "dg_k"], label="cfg3[b=0] ")
+
+
+def test_cfg4_long_context_extras_full_size(gpu_device):
+    _slice_check(gpu_device, CONFIGS[4], [(1, 3)], odtype=torch.float32)
+
+
+def test_cfg5_wide_head_full_size(gpu_device):
+    _slice_check(gpu_device, CONFIGS[5], [(0, 0), (3, 3)])
+
+
+def test_backward_is_deterministic(gpu_device):
+    x = gen(2, 6, 2, 512, 512, 64, BF16, extras=True, seed=4)
+    a = run_gpu(x, gpu_device)
+    b = run_gpu(x, gpu_device)
+    for n in a:
+        assert torch.equal(a[n], b[n]), n
+
+
+# ------------------------------------------------------------------ the reference's call signature
+
+
+def _flat(x, H):
+    return orc.flatten_heads(x).contiguous()
+
+
+def test_dropin_matches_live_module_variant_a(gpu_device):
+    """Positional call exactly as the reference makes it (expanded K/V, scalar gain): compare with the
+    restatement of the live module, attention.py:43-80, incl. its bf16 rounding points."""
+    B, H, Hkv, S, D = 2, 6, 2, 320, 64
+    x = gen(B, H, Hkv, S, S, D, BF16, scalar_gain=True, no_gk=True, seed=7)
+    Q = _flat(x["q"], H)
+    K = orc.expand_kv_flat(_flat(x["k"], Hkv), Hkv, H).contiguous()
+    V = orc.expand_kv_flat(_flat(x["v"], Hkv), Hkv, H).contiguous()
+    gain = x["g_q"]
+    dO = _flat(x["d_o"], H)
+    # reference side (CPU): bf16 module forward; gradients from the fp32 evaluation of the same formula
+    ref_out = orc.live_module_variant_a(Q, K, V, gain)
+    Qr, Kr, Vr, gr = (t.detach().clone().float().requires_grad_(True) for t in (Q, K, V, gain))
+    orc.live_module_variant_a(Qr, Kr, Vr, gr).backward(dO.float())
+    Qd, Kd, Vd, gd = (t.detach().clone().to(gpu_device).requires_grad_(True) for t in (Q, K, V, gain))
+    out = QKNormFlashAttnFunc.apply(Qd, Kd, Vd, gd, True, 0)
+    assert out.shape == Q.shape and out.dtype == Q.dtype
+    out.backward(dO.to(gpu_device))
+    got = {"y": out.detach().cpu(), "dq": Qd.grad.cpu(), "dk": Kd.grad.cpu(), "dv": Vd.grad.cpu(), "dg": gd.grad.cpu()}
+    ref = {"y": ref_out, "dq": Qr.grad, "dk": Kr.grad, "dv": Vr.grad, "dg": gr.grad}
+    assert gd.grad.shape == gain.shape and gd.grad.dtype == gain.dtype
+    xs = dict(x, g_k=None)
+    compare(got, ref, BF16, scales={"dg": scalar_gain_scale(xs)["dg_q"]})
+
+
+def test_dropin_gqa_native_equals_expanded_and_2d_inputs(gpu_device):
+    B, H, Hkv, S, D = 2, 6, 2, 192, 64
+    x = gen(B, H, Hkv, S, S, D, BF16, scalar_gain=True, no_gk=True, seed=8)
+    Q, K, V = _flat(x["q"], H), _flat(x["k"], Hkv), _flat(x["v"], Hkv)
+    Kx, Vx = (orc.expand_kv_flat(t, Hkv, H).contiguous() for t in (K, V))
+    d = gpu_device
+    g = x["g_q"].to(d)
+    o_exp = QKNormFlashAttnFunc.apply(Q.to(d), Kx.to(d), Vx.to(d), g)
+    o_nat = QKNormFlashAttnFunc.apply(Q.to(d), K.to(d), V.to(d), g, True, 0, None, None, None, None, 2.0, Hkv)
+    assert torch.equal(o_exp, o_nat)
+    o2 = QKNormFlashAttnFunc.apply(Q[0].to(d), Kx[0].to(d), Vx[0].to(d), g)
+    assert o2.shape == (1, S, D) and torch.equal(o2[0], o_exp[0])
+
+
+def test_dropin_rejects_bad_inputs(gpu_device):
+    d = gpu_device
+    Q = torch.randn(2, 64, 64, device=d, dtype=BF16)
+    g = torch.ones(1, device=d)
+    with pytest.raises(AssertionError):
+        QKNormFlashAttnFunc.apply(Q.transpose(0, 1), Q, Q, g)       # not contiguous
+    with pytest.raises(AssertionError):
+        QKNormFlashAttnFunc.apply(Q.cpu(), Q.cpu(), Q.cpu(), g)     # not on the device
+    with pytest.raises(TypeError):
+        QKNormFlashAttnFunc.apply(Q.half(), Q.half(), Q.half(), g)  # unsupported dtype
+    with pytest.raises(RuntimeError, match="head_dim"):
+        QKNormFlashAttnFunc.apply(Q[..., :48].contiguous(), Q[..., :48].contiguous(), Q[..., :48].contiguous(), g)
+
+
+def test_fused_triton_formula_is_reachable_variant_b(gpu_device):
+    """eps = 1e-8/d, sm_scale = 1/d reproduces the fused Triton kernel's own logits (gain*cos)."""
+    S, D = 128, 64
+    x = gen(3, 1, 1, S, S, D, F32, scalar_gain=True, no_gk=True, seed=9)
+    Q, K, V = (x[n][:, 0].contiguous() for n in ("q", "k", "v"))
+    O_ref, L_ref = orc.fused_kernel_variant_b(Q.double(), K.double(), V.double(), x["g_q"].double())
+    eps, sc = orc.family_params("B", D)
+    d = gpu_device
+    out = QKNormFlashAttnFunc.apply(Q.to(d), K.to(d), V.to(d), x["g_q"].to(d), True, 0, None, None, None, None, 2.0, None, eps, sc)
+    compare({"y": out.cpu()}, {"y": O_ref}, F32)
+
+
+def test_module_state_dict_and_forward(gpu_device):
+    m = SelfDotProductAttnQKNorm(64).to(gpu_device)
+    assert list(m.state_dict().keys()) == ["gain"] and m.gain.shape == (1,) and m.gain.dtype == torch.float32
+    x = gen(1, 4, 4, 96, 96, 64, BF16, seed=10)
+    Q, K, V = (_flat(x[n], 4).to(gpu_device) for n in ("q", "k", "v"))
+    out = m(Q, K, V, True, q_start=0)
+    ref = orc.live_module_variant_a(Q.cpu(), K.cpu(), V.cpu(), torch.ones(1))
+    compare({"y": out.cpu()}, {"y": ref}, BF16)
+
+
+def test_strided_projection_views(gpu_device):
+    """q/k/v taken as strided slices of one `[b, S, (H+2Hkv)*D]` projection output (no copies)."""
+    B, H, Hkv, S, D = 2, 6, 2, 160, 64
+    x = gen(B, H, Hkv, S, S, D, BF16, seed=11)
+    W = (H + 2 * Hkv) * D
+    proj = torch.empty(B, S, W, dtype=BF16)
+    proj[..., : H * D] = x["q"].permute(0, 2, 1, 3).reshape(B, S, H * D)
+    proj[..., H * D: (H + Hkv) * D] = x["k"].permute(0, 2, 1, 3).reshape(B, S, Hkv * D)
+    proj[..., (H + Hkv) * D:] = x["v"].permute(0, 2, 1, 3).reshape(B, S, Hkv * D)
+    pd = proj.to(gpu_device)
+    q = pd[..., : H * D].view(B, S, H, D).permute(0, 2, 1, 3)
+    k = pd[..., H * D: (H + Hkv) * D].view(B, S, Hkv, D).permute(0, 2, 1, 3)
+    v = pd[..., (H + Hkv) * D:].view(B, S, Hkv, D).permute(0, 2, 1, 3)
+    y = qknorm_attention(q, k, v, x["g_q"].to(gpu_device), x["g_k"].to(gpu_device))
+    ref = run_oracle(x, backward=False)
+    compare({"y": y.cpu()}, ref, BF16, names=["y"])
