@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused QK-norm flash attention hot path on one MI355X.
+
+A step = one forward + one backward of the attention op over one batch of synthetic input, already
+resident in HBM, enqueued through the C ABI (segpt_attn_fwd + the four stages of segpt_attn_bwd, in
+order, on torch's current stream).  Prints ONE JSON line:
+
+  value      whole-step algorithmic TFLOP/s: (2 + 5) * B*H*S^2*D / step time (causal FlashAttention
+             convention; norm/softmax/gate/mix work and recomputation are not credited)
+  roofline   the slowest kernel of the step: its credited FLOPs / its average duration, measured
+             with HIP events recorded on the launch stream inside the timed region, vs the MI355X
+             dense bf16 MFMA peak
+  cpu_baseline  the CPU restatement of the reference's live path (fp32 RMS-normalise ->
+             scaled_dot_product_attention(is_causal) -> autograd backward) timed on this host on a
+             bounded sample of the same workload
+
+    python bench.py [--gpus 1] [--steps 50] [--warmup 10] [--cfg 3] [--no-cpu-baseline]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MI355X_BF16_DENSE_TFLOPS = 2516.6  # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz (vendor dense figure, no sparsity)
+MI355X_HBM_GBS = 8000.0
+
+
+def cpu_baseline(c, batches: int):
+    """Times the oracle's SDPA form of the reference's live path on the host cores (fp32)."""
+    import torch
+
+    from oracle import qknorm_attn_oracle as orc
+    from sample_efficient_gpt_amd import make_inputs
+
+    cs = c.scaled(B=batches)
+    x = make_inputs(cs)
+    f = lambda n: x[n].float()
+    q, k, v = (f(n).requires_grad_(c.backward) for n in ("q", "k", "v"))
+    gq, gk = (f(n).requires_grad_(c.backward) for n in ("g_q", "g_k"))
+    t0 = time.perf_counter()
+    y = orc.attention_forward_sdpa(q, k, v, gq, gk, eps=cs.eps, sm_scale=cs.sm_scale)
+    if c.backward:
+        y.backward(f("d_o"))
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(cs.flops() / dt / 1e12, 5),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{batches} of {c.B} batches of the same workload, fp32, one cold run of fwd{'+bwd' if c.backward else ''} "
+                  f"({dt:.2f} s): RMS-normalise + F.scaled_dot_product_attention(is_causal) + autograd",
+        "seconds": round(dt, 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--cfg", type=int, default=3, help="benchmark configuration (3 = IMU-1 shape fwd+bwd, the headline)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-batches", type=int, default=2)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU only (the attention path has no cross-GPU step); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from sample_efficient_gpt_amd import CONFIGS, make_inputs
+    from sample_efficient_gpt_amd.plan import AttnPlan
+
+    c = CONFIGS[args.cfg]
+    if c.dtype != torch.bfloat16 and args.cfg != 1:
+        raise SystemExit("unsupported config")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    x = make_inputs(c, device=dev)
+    plan = AttnPlan(x, eps=c.eps, sm_scale=c.sm_scale, gate_scale=c.gate_scale, backward=c.backward)
+    names = ["fwd"] + (["bwd_pre", "bwd_dkdv", "bwd_dq", "bwd_reduce"] if c.backward else [])
+
+    def step(events=None):
+        if events is not None:
+            events[0].record()
+        plan.forward()
+        if events is not None:
+            events[1].record()
+        if c.backward:
+            for s in range(4):
+                plan.backward_stage(s)
+                if events is not None:
+                    events[2 + s].record()
+
+    for _ in range(args.warmup):
+        step()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    kern_ms = {n: sum(e[j].elapsed_time(e[j + 1]) for e in evs) / args.steps for j, n in enumerate(names)}
+
+    # cross-check: the plain entry points (segpt_attn_fwd + segpt_attn_bwd), no events in between
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.forward()
+        if c.backward:
+            plan.backward()
+    torch.cuda.synchronize()
+    ms_plain = (time.perf_counter() - t1) / args.steps * 1e3
+
+    unit = c.B * c.H * c.S * c.S * c.D  # one causal S x S x D contraction, in FLOPs
+    credited = {"fwd": 2 * unit, "bwd_dkdv": 4 * unit, "bwd_dq": 1 * unit}  # dq's recomputed S and dP are not credited
+    total_flops = c.flops()
+    value = total_flops / (ms_per_step * 1e-3) / 1e12
+    dom = max((n for n in names if n in credited), key=lambda n: kern_ms[n])
+    achieved = credited[dom] / (kern_ms[dom] * 1e-3) / 1e12
+    elem = 2
+    hbm_bytes = {  # algorithmic bytes of the HBM-bound helpers
+        "bwd_pre": c.B * c.H * c.S * (2 * c.D * elem + 4) + (c.B * c.H * c.S * (c.D * elem + 2 * elem) if c.extras else 0),
+    }
+    kernels = {}
+    for n in names:
+        k = {"ms": round(kern_ms[n], 5)}
+        if n in credited:
+            k["credited_tflops"] = round(credited[n] / (kern_ms[n] * 1e-3) / 1e12, 2)
+            k["frac_of_bf16_peak"] = round(k["credited_tflops"] / MI355X_BF16_DENSE_TFLOPS, 4)
+        if n in hbm_bytes:
+            k["algorithmic_GBps"] = round(hbm_bytes[n] / (kern_ms[n] * 1e-3) / 1e9, 1)
+        kernels[n] = k
+
+    out = {
+        "metric": "attention fwd+bwd TFLOP/s at IMU-1 shape, 1 GPU" if args.cfg == 3 else f"attention TFLOP/s, cfg {args.cfg}",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if c.dtype == torch.bfloat16 else "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"cfg{c.cfg} {c.name}: B={c.B} S={c.S} q_heads={c.H} kv_heads={c.Hkv} head_dim={c.D} causal "
+                        f"QK-norm (vector scales, eps 1e-6){' + per-head gate + value residual' if c.extras else ''}, "
+                        f"{'forward + backward' if c.backward else 'forward only'}",
+            "algorithmic_flops_per_step": total_flops,
+        },
+        "pct_of_bf16_mfma_peak": round(100 * value / MI355X_BF16_DENSE_TFLOPS, 2),
+        "ms_per_step_plain_entry_points": round(ms_plain, 5),
+        "roofline": {
+            "kernel": dom,
+            "bound": "mfma",
+            "achieved": round(achieved, 2),
+            "peak": MI355X_BF16_DENSE_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / MI355X_BF16_DENSE_TFLOPS, 4),
+            "traffic": None,
+            "credited_flops_per_launch": credited[dom],
+            "avg_launch_ms": round(kern_ms[dom], 5),
+        },
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(c, min(args.cpu_batches, c.B))
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libsegpt_attn.so")
 SEGPT_ABI_VERSION = 1
 SEGPT_DTYPE_BF16 = 0
 SEGPT_DTYPE_FP32 = 1
+BWD_STAGES = ("pre", "dkdv", "dq", "reduce")  # SEGPT_BWD_STAGE_* = index
 
 EXPORTED_SYMBOLS = (
     "segpt_abi_version",
@@ -22,6 +23,7 @@ EXPORTED_SYMBOLS = (
     "segpt_attn_workspace_bytes",
     "segpt_attn_fwd",
     "segpt_attn_bwd",
+    "segpt_attn_bwd_stage",
 )
 
 
@@ -91,6 +93,8 @@ def load():
         lib.segpt_attn_fwd.argtypes = [C.POINTER(AttnParams), C.c_void_p]
         lib.segpt_attn_bwd.restype = C.c_int
         lib.segpt_attn_bwd.argtypes = [C.POINTER(AttnParams), C.c_void_p]
+        lib.segpt_attn_bwd_stage.restype = C.c_int
+        lib.segpt_attn_bwd_stage.argtypes = [C.POINTER(AttnParams), C.c_int, C.c_void_p]
         ver = lib.segpt_abi_version()
         if ver != SEGPT_ABI_VERSION:
             raise RuntimeError(f"libsegpt_attn.so ABI version {ver}, binding expects {SEGPT_ABI_VERSION}")

@@ -125,6 +125,7 @@ const char* segpt_strerror(int code) {
     case SEGPT_E_EXTRAS: return "inconsistent optional operands (v_first/vr_coef/gate and their gradient slots)";
     case SEGPT_E_QSTART: return "q_start must be >= 0";
     case SEGPT_E_ALIGN: return "a base pointer is not 16-byte aligned (workspace: 256-byte)";
+    case SEGPT_E_STAGE: return "unknown backward stage (expected SEGPT_BWD_STAGE_*)";
     default: return code > 0 ? "HIP runtime error raised by a kernel launch" : "unknown segpt error code";
   }
 }
@@ -146,7 +147,7 @@ int segpt_attn_fwd(const segpt_attn_params* p, void* stream) {
   return p->dtype == SEGPT_DTYPE_FP32 ? launch_fwd_f32(a, st) : launch_fwd_bf16(a, st);
 }
 
-int segpt_attn_bwd(const segpt_attn_params* p, void* stream) {
+static int bwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi, void* stream) {
   int rc = check_common(p);
   if (rc) return rc;
   if ((rc = check_bwd(p))) return rc;
@@ -161,10 +162,27 @@ int segpt_attn_bwd(const segpt_attn_params* p, void* stream) {
   a.n_dq_blocks = dq_blocks(*p);
   a.n_dkdv_blocks = dkdv_blocks(*p);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if ((rc = launch_bwd_pre(a, st))) return rc;
-  rc = p->dtype == SEGPT_DTYPE_FP32 ? launch_bwd_f32(a, st) : launch_bwd_bf16(a, st);
-  if (rc) return rc;
-  return launch_bwd_reduce(a, st);
+  const bool f32 = p->dtype == SEGPT_DTYPE_FP32;
+  for (int stage = stage_lo; stage <= stage_hi; ++stage) {
+    switch (stage) {
+      case SEGPT_BWD_STAGE_PRE: rc = launch_bwd_pre(a, st); break;
+      case SEGPT_BWD_STAGE_DKDV: rc = f32 ? launch_bwd_dkdv_f32(a, st) : launch_bwd_dkdv_bf16(a, st); break;
+      case SEGPT_BWD_STAGE_DQ: rc = f32 ? launch_bwd_dq_f32(a, st) : launch_bwd_dq_bf16(a, st); break;
+      case SEGPT_BWD_STAGE_REDUCE: rc = launch_bwd_reduce(a, st); break;
+      default: return SEGPT_E_STAGE;
+    }
+    if (rc) return rc;
+  }
+  return SEGPT_OK;
+}
+
+int segpt_attn_bwd(const segpt_attn_params* p, void* stream) {
+  return bwd_stage_impl(p, SEGPT_BWD_STAGE_PRE, SEGPT_BWD_STAGE_REDUCE, stream);
+}
+
+int segpt_attn_bwd_stage(const segpt_attn_params* p, int stage, void* stream) {
+  if (stage < SEGPT_BWD_STAGE_PRE || stage > SEGPT_BWD_STAGE_REDUCE) return SEGPT_E_STAGE;
+  return bwd_stage_impl(p, stage, stage, stream);
 }
 
 }  // extern "C"

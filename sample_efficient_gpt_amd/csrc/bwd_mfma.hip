@@ -529,19 +529,24 @@ __global__ __launch_bounds__(kThreadsM) void bwd_dkdv_bf16_kernel(KArgs a) {
 }
 
 template <int D>
-int launch_bwd_t(const KArgs& a, hipStream_t st) {
+int launch_dkdv_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
-  constexpr int NQB = BwdCfg<D>::kNQB, NKB = BwdCfg<D>::kNKB;
-  const int n_qt = (p.Sq + 128 * NQB - 1) / (128 * NQB);
+  constexpr int NKB = BwdCfg<D>::kNKB;
   const int n_kvt = (p.Sk + 128 * NKB - 1) / (128 * NKB);
-  dim3 gq((unsigned)(n_qt * p.H * p.B)), gk((unsigned)(n_kvt * p.Hkv * p.B)), block(kThreadsM);
-  if (p.v_first.ptr) {
-    hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D, NKB, true>), gk, block, 0, st, a);
-    hipLaunchKernelGGL((bwd_dq_bf16_kernel<D, NQB, true>), gq, block, 0, st, a);
-  } else {
-    hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D, NKB, false>), gk, block, 0, st, a);
-    hipLaunchKernelGGL((bwd_dq_bf16_kernel<D, NQB, false>), gq, block, 0, st, a);
-  }
+  dim3 gk((unsigned)(n_kvt * p.Hkv * p.B)), block(kThreadsM);
+  if (p.v_first.ptr) hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D, NKB, true>), gk, block, 0, st, a);
+  else hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D, NKB, false>), gk, block, 0, st, a);
+  return (int)hipGetLastError();
+}
+
+template <int D>
+int launch_dq_t(const KArgs& a, hipStream_t st) {
+  const segpt_attn_params& p = a.p;
+  constexpr int NQB = BwdCfg<D>::kNQB;
+  const int n_qt = (p.Sq + 128 * NQB - 1) / (128 * NQB);
+  dim3 gq((unsigned)(n_qt * p.H * p.B)), block(kThreadsM);
+  if (p.v_first.ptr) hipLaunchKernelGGL((bwd_dq_bf16_kernel<D, NQB, true>), gq, block, 0, st, a);
+  else hipLaunchKernelGGL((bwd_dq_bf16_kernel<D, NQB, false>), gq, block, 0, st, a);
   return (int)hipGetLastError();
 }
 
@@ -550,9 +555,15 @@ int launch_bwd_t(const KArgs& a, hipStream_t st) {
 int bf16_dq_rows_per_block(int D) { return D == 64 ? 128 * BwdCfg<64>::kNQB : 128 * BwdCfg<128>::kNQB; }
 int bf16_dkdv_rows_per_block(int D) { return D == 64 ? 128 * BwdCfg<64>::kNKB : 128 * BwdCfg<128>::kNKB; }
 
-int launch_bwd_bf16(const KArgs& a, hipStream_t st) {
-  if (a.p.D == 64) return launch_bwd_t<64>(a, st);
-  if (a.p.D == 128) return launch_bwd_t<128>(a, st);
+int launch_bwd_dkdv_bf16(const KArgs& a, hipStream_t st) {
+  if (a.p.D == 64) return launch_dkdv_t<64>(a, st);
+  if (a.p.D == 128) return launch_dkdv_t<128>(a, st);
+  return (int)hipErrorInvalidValue;
+}
+
+int launch_bwd_dq_bf16(const KArgs& a, hipStream_t st) {
+  if (a.p.D == 64) return launch_dq_t<64>(a, st);
+  if (a.p.D == 128) return launch_dq_t<128>(a, st);
   return (int)hipErrorInvalidValue;
 }
 

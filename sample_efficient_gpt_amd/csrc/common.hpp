@@ -92,9 +92,11 @@ __device__ __forceinline__ float sigmoidf_acc(float z) { return 1.0f / (1.0f + e
 
 // host-side launchers (one per translation unit); each returns a hipError_t as int
 int launch_fwd_f32(const KArgs& a, hipStream_t st);
-int launch_bwd_f32(const KArgs& a, hipStream_t st);
+int launch_bwd_dkdv_f32(const KArgs& a, hipStream_t st);
+int launch_bwd_dq_f32(const KArgs& a, hipStream_t st);
 int launch_fwd_bf16(const KArgs& a, hipStream_t st);
-int launch_bwd_bf16(const KArgs& a, hipStream_t st);
+int launch_bwd_dkdv_bf16(const KArgs& a, hipStream_t st);
+int launch_bwd_dq_bf16(const KArgs& a, hipStream_t st);
 int launch_bwd_pre(const KArgs& a, hipStream_t st);     // delta, dgate, do_eff
 int launch_bwd_reduce(const KArgs& a, hipStream_t st);  // dg_q, dg_k, dvr_coef from the partials
 

@@ -473,22 +473,25 @@ int launch_fwd_f32(const KArgs& a, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
-int launch_bwd_f32(const KArgs& a, hipStream_t st) {
+int launch_bwd_dq_f32(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
-  dim3 gq((p.Sq + kRows - 1) / kRows, p.H, p.B), gk((p.Sk + kRows - 1) / kRows, p.Hkv, p.B), block(kThreads);
+  dim3 gq((p.Sq + kRows - 1) / kRows, p.H, p.B), block(kThreads);
   switch (p.D) {
-    case 32:
-      hipLaunchKernelGGL(bwd_dq_f32_kernel<32>, gq, block, 0, st, a);
-      hipLaunchKernelGGL(bwd_dkdv_f32_kernel<32>, gk, block, 0, st, a);
-      break;
-    case 64:
-      hipLaunchKernelGGL(bwd_dq_f32_kernel<64>, gq, block, 0, st, a);
-      hipLaunchKernelGGL(bwd_dkdv_f32_kernel<64>, gk, block, 0, st, a);
-      break;
-    case 128:
-      hipLaunchKernelGGL(bwd_dq_f32_kernel<128>, gq, block, 0, st, a);
-      hipLaunchKernelGGL(bwd_dkdv_f32_kernel<128>, gk, block, 0, st, a);
-      break;
+    case 32: hipLaunchKernelGGL(bwd_dq_f32_kernel<32>, gq, block, 0, st, a); break;
+    case 64: hipLaunchKernelGGL(bwd_dq_f32_kernel<64>, gq, block, 0, st, a); break;
+    case 128: hipLaunchKernelGGL(bwd_dq_f32_kernel<128>, gq, block, 0, st, a); break;
+    default: return (int)hipErrorInvalidValue;
+  }
+  return (int)hipGetLastError();
+}
+
+int launch_bwd_dkdv_f32(const KArgs& a, hipStream_t st) {
+  const segpt_attn_params& p = a.p;
+  dim3 gk((p.Sk + kRows - 1) / kRows, p.Hkv, p.B), block(kThreads);
+  switch (p.D) {
+    case 32: hipLaunchKernelGGL(bwd_dkdv_f32_kernel<32>, gk, block, 0, st, a); break;
+    case 64: hipLaunchKernelGGL(bwd_dkdv_f32_kernel<64>, gk, block, 0, st, a); break;
+    case 128: hipLaunchKernelGGL(bwd_dkdv_f32_kernel<128>, gk, block, 0, st, a); break;
     default: return (int)hipErrorInvalidValue;
   }
   return (int)hipGetLastError();

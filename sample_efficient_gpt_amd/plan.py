@@ -1,0 +1,63 @@
+"""Pre-bound launch plan: one filled `segpt_attn_params` plus every output / workspace buffer, so that a
+tight loop (benchmark, serving) makes C-ABI calls without building structs or allocating per call."""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+from .function import _fill_common
+
+
+class AttnPlan:
+    """Binds canonical-layout tensors (q [B,H,S,D], k/v [B,Hkv,S,D], ...) once; `forward()`,
+    `backward()` and `backward_stage(i)` then only enqueue kernels on the current stream."""
+
+    def __init__(self, x: dict, *, eps=1e-6, sm_scale=None, gate_scale=2.0, causal=True, q_start=0, backward=True):
+        self.lib = _lib.load()
+        q, k, v = x["q"], x["k"], x["v"]
+        dev = q.device
+        self.x = x
+        f32 = lambda t: None if t is None else t.detach().to(device=dev, dtype=torch.float32).reshape(-1).contiguous()
+        self.g_q, self.g_k, self.coef = f32(x["g_q"]), f32(x.get("g_k")), f32(x.get("vr_coef"))
+        self.v_first, self.gate = x.get("v_first"), x.get("gate_logits")
+        B, H, Sq, D = q.shape
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(D)
+        self.y = torch.empty_like(q)
+        self.lse = torch.empty((B, H, Sq), dtype=torch.float32, device=dev)
+        p = _lib.new_params()
+        _fill_common(p, q, k, v, self.y, self.lse, self.g_q, self.g_k, self.v_first, self.coef, self.gate, gate_scale,
+                     eps, sm_scale, causal, q_start)
+        self.p = p
+        self.has_bwd = backward
+        if backward:
+            self.d_o = x["d_o"]
+            self.dq, self.dk, self.dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+            self.dv_first = None if self.v_first is None else torch.empty_like(self.v_first)
+            self.dgate = None if self.gate is None else torch.empty_like(self.gate)
+            self.dg_q = torch.empty_like(self.g_q)
+            self.dg_k = None if self.g_k is None else torch.empty_like(self.g_k)
+            self.dcoef = None if self.coef is None else torch.empty(2, dtype=torch.float32, device=dev)
+            p.d_o, p.dq, p.dk, p.dv = _lib.t4(self.d_o), _lib.t4(self.dq), _lib.t4(self.dk), _lib.t4(self.dv)
+            p.dv_first, p.dgate = _lib.t4(self.dv_first), _lib.t3(self.dgate)
+            p.dg_q, p.dg_k, p.dvr_coef = _lib.ptr(self.dg_q), _lib.ptr(self.dg_k), _lib.ptr(self.dcoef)
+            nbytes = max(int(self.lib.segpt_attn_workspace_bytes(p, 1)), 256)
+            self.ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            p.workspace, p.workspace_bytes = self.ws.data_ptr(), nbytes
+        self.stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def _chk(self, rc, what):
+        if rc != 0:
+            raise _lib.SegptError(rc, what)
+
+    def forward(self):
+        self._chk(self.lib.segpt_attn_fwd(self.p, self.stream), "segpt_attn_fwd")
+
+    def backward(self):
+        self._chk(self.lib.segpt_attn_bwd(self.p, self.stream), "segpt_attn_bwd")
+
+    def backward_stage(self, stage: int):
+        self._chk(self.lib.segpt_attn_bwd_stage(self.p, stage, self.stream), "segpt_attn_bwd_stage")
