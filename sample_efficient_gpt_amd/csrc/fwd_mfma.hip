@@ -1,6 +1,7 @@
 // bf16 forward: causal GQA flash attention with the QK RMS-norm fused into the tile loads.
 //
-// Workgroup = 4 waves; wave w owns NQB blocks of 32 queries.  Scores are produced TRANSPOSED,
+// Workgroup = 4 waves (two workgroups share a CU so that one's softmax overlaps the other's MFMAs);
+// wave w owns NQB blocks of 32 queries.  Scores are produced TRANSPOSED,
 //   S^T[key][query] = Khat[key][:] . Qhat[query][:]          (A = Khat tile from LDS, B = Qhat registers)
 // so every lane owns one query column: the online-softmax state (m, l) and the rescale factor are
 // per-lane scalars, row reductions are in-register plus one exchange with lane^32, and the bf16
@@ -19,8 +20,27 @@ struct FwdCfg {
   static constexpr int kBQ = 4 * 32 * NQB;  // queries per workgroup
 };
 
+// Largest |log2-unit logit| the normalised operands can produce: |Qhat.Khat| <= |Qhat| |Khat| with
+// |Khat| <= sqrt(D) and |Qhat| <= sm_scale*log2e*sqrt(D)*max|g_q g_k|.  When it is small the softmax needs
+// no running maximum at all (softmax is shift invariant and exp2 cannot overflow): P = exp2(S2) directly.
+__device__ __forceinline__ float logit_bound(const segpt_attn_params& p, int lane) {
+  float gm = 0.f;
+  for (int d = lane; d < p.D; d += 64) {
+    float g = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
+    if (p.gk_numel == 1) g *= p.g_k[0];
+    else if (p.gk_numel > 1) g *= p.g_k[d];
+    gm = fmaxf(gm, fabsf(g));
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) gm = fmaxf(gm, __shfl_xor(gm, o, 64));
+  return p.sm_scale * kLog2e * (float)p.D * gm * 1.02f;
+}
+
+constexpr float kNoMaxBound = 64.f;   // |S2| below this: P in [2^-64, 2^64], sums stay far inside fp32 range
+constexpr float kLazyThresh = 16.f;   // general path: the subtracted reference is raised only when exceeded by 2^16
+
 template <int D, int NQB, bool VR>
-__global__ __launch_bounds__(kThreadsM) void fwd_bf16_kernel(KArgs a) {
+__global__ __launch_bounds__(kThreadsM, 2) void fwd_bf16_kernel(KArgs a) {
   using T = Tile<D>;
   constexpr int BQ = FwdCfg<D, NQB>::kBQ;
   constexpr int KS = D / 16;  // contraction steps of QK^T
@@ -39,6 +59,7 @@ __global__ __launch_bounds__(kThreadsM) void fwd_bf16_kernel(KArgs a) {
 
   float c1 = 1.f, c2 = 0.f;
   if (VR) { c1 = p.vr_coef[0]; c2 = p.vr_coef[1]; }
+  const bool bounded = logit_bound(p, lane) <= kNoMaxBound;  // wave-uniform
 
   // ---- Qhat registers: B operands of S^T, [nb][ks]
   bf16x8 qreg[NQB][KS];
@@ -78,9 +99,11 @@ __global__ __launch_bounds__(kThreadsM) void fwd_bf16_kernel(KArgs a) {
     for (int nb = 0; nb < NQB; ++nb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) oacc[mb][nb][r] = 0.f;
-  float m_run[NQB], l_run[NQB];
+  // m_ref: the value subtracted from the logits before exp2 (0 on the bounded path); l_run: this lane's
+  // share of the row sum (its half of the keys; halves are added in the epilogue)
+  float m_ref[NQB], l_run[NQB];
 #pragma unroll
-  for (int nb = 0; nb < NQB; ++nb) { m_run[nb] = -INFINITY; l_run[nb] = 0.f; }
+  for (int nb = 0; nb < NQB; ++nb) { m_ref[nb] = bounded ? 0.f : -INFINITY; l_run[nb] = 0.f; }
 
   int kend = p.Sk;
   if (p.causal) kend = min(p.Sk, q0 + BQ + p.q_start);
@@ -98,77 +121,75 @@ __global__ __launch_bounds__(kThreadsM) void fwd_bf16_kernel(KArgs a) {
     const bool more = jt + 1 < n_kt;
     if (more) stage_load<D, VR>(p, b, g, j0 + kBK, sr);
 
-    // wave-uniform: does this wave see any key of the tile?
-    const bool active = !p.causal || j0 <= qw0 + 32 * NQB - 1 + p.q_start;
-    if (active) {
-      f32x16 s[2][NQB];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < 2; ++kb) {
+      const int jb = j0 + 32 * kb;  // first key of this 32-key block
+      // wave-uniform: does this wave see any key of the block?
+      const bool active = jb < p.Sk && (!p.causal || jb <= qw0 + 32 * NQB - 1 + p.q_start);
+      if (active) {
+        f32x16 s[NQB];
 #pragma unroll
         for (int nb = 0; nb < NQB; ++nb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) s[kb][nb][r] = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+          for (int r = 0; r < 16; ++r) s[nb][r] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const bf16x8 af = frag_rowmajor<D>(kt, kb, ks, lane);
 #pragma unroll
-          for (int nb = 0; nb < NQB; ++nb) s[kb][nb] = mfma32(af, qreg[nb][ks], s[kb][nb]);
+          for (int nb = 0; nb < NQB; ++nb) s[nb] = mfma32(af, qreg[nb][ks], s[nb]);
         }
-      const bool need_mask = (p.causal && j0 + kBK - 1 > qw0 + p.q_start) || j0 + kBK > p.Sk;
-      if (need_mask) {
+        const bool need_mask = (p.causal && jb + 31 > qw0 + p.q_start) || jb + 32 > p.Sk;
+        if (need_mask) {
 #pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) {
-          const int qlim = p.causal ? min(qw0 + 32 * nb + ln + p.q_start, p.Sk - 1) : p.Sk - 1;
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
+          for (int nb = 0; nb < NQB; ++nb) {
+            const int qlim = p.causal ? min(qw0 + 32 * nb + ln + p.q_start, p.Sk - 1) : p.Sk - 1;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              const int key = j0 + 32 * kb + 8 * (r >> 2) + 4 * hh + (r & 3);
-              if (key > qlim) s[kb][nb][r] = -INFINITY;
+              const int key = jb + 8 * (r >> 2) + 4 * hh + (r & 3);
+              if (key > qlim) s[nb][r] = -INFINITY;
             }
-        }
-      }
-      bf16x8 pb[2][2][NQB];
-#pragma unroll
-      for (int nb = 0; nb < NQB; ++nb) {
-        float mx = m_run[nb];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][nb][r]);
-        mx = half_max(mx);
-        const float corr = fast_exp2(m_run[nb] - mx);
-        m_run[nb] = mx;
-        float ps = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float e = fast_exp2(s[kb][nb][r] - mx);
-            s[kb][nb][r] = e;
-            ps += e;
           }
-          pb[kb][0][nb] = pack_c_half(s[kb][nb], 0);
-          pb[kb][1][nb] = pack_c_half(s[kb][nb], 1);
         }
-        l_run[nb] = l_run[nb] * corr + ps;
+        if (!bounded) {
+          // general path: lazily maintained reference, raised only when a row exceeds it by 2^kLazyThresh
+#pragma unroll
+          for (int nb = 0; nb < NQB; ++nb) {
+            float mx = s[nb][0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[nb][r]);
+            mx = half_max(mx);
+            const bool need = mx > m_ref[nb] + kLazyThresh;
+            if (__builtin_amdgcn_ballot_w64(need) != 0) {
+              const float m_new = need ? mx : m_ref[nb];
+              const float corr = fast_exp2(m_ref[nb] - m_new);
+              m_ref[nb] = m_new;
+              l_run[nb] *= corr;
+#pragma unroll
+              for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[mb][nb][r] *= corr;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[nb][r] -= m_ref[nb];
+          }
+        }
+        bf16x8 pb[2][NQB];
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) s[nb][r] = fast_exp2(s[nb][r]);
+          pb[0][nb] = pack_c_half_sum(s[nb], 0, l_run[nb]);
+          pb[1][nb] = pack_c_half_sum(s[nb], 1, l_run[nb]);
+        }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[mb][nb][r] *= corr;
-      }
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2) {
             const bf16x8 vf = frag_transposed<D>(vt, mb, 2 * kb + s2, lane);
 #pragma unroll
-            for (int nb = 0; nb < NQB; ++nb) oacc[mb][nb] = mfma32(vf, pb[kb][s2][nb], oacc[mb][nb]);
+            for (int nb = 0; nb < NQB; ++nb) oacc[mb][nb] = mfma32(vf, pb[s2][nb], oacc[mb][nb]);
           }
+      }
     }
     if (more) {
       uint16_t* nk = lds + ((jt + 1) & 1) * 2 * T::kElems;
@@ -189,7 +210,7 @@ __global__ __launch_bounds__(kThreadsM) void fwd_bf16_kernel(KArgs a) {
       const float z = bf16_to_f32(reinterpret_cast<const uint16_t*>(p.gate.ptr)[(int64_t)b * p.gate.stride_b + (int64_t)rc * p.gate.stride_s + (int64_t)h * p.gate.stride_h]);
       f *= p.gate_scale / (1.0f + __expf(-z));
     }
-    if (live && hh == 0) p.lse[((int64_t)b * p.H + h) * p.Sq + row] = (m_run[nb] + __log2f(l)) * kLn2;
+    if (live && hh == 0) p.lse[((int64_t)b * p.H + h) * p.Sq + row] = (m_ref[nb] + __log2f(l)) * kLn2;
     uint16_t* op = live ? row_ptr_mut<uint16_t>(p.o, b, h, row) : nullptr;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {

@@ -52,12 +52,29 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float fast_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
-// sum over the kTPR adjacent lanes that stage one row
+// x + (x of another lane) through a DPP lane pattern (no LDS traffic, fuses into v_add_f32_dpp)
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+  return x + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+
+// sum over the kTPR (8 or 16) adjacent lanes that stage one row; every lane of the group gets the total
 template <int TPR>
 __device__ __forceinline__ float row_group_sum(float x) {
-#pragma unroll
-  for (int o = 1; o < TPR; o <<= 1) x += __shfl_xor(x, o, 64);
+  static_assert(TPR == 8 || TPR == 16, "row groups are 8 or 16 lanes");
+  x = dpp_add<0xB1>(x);   // quad_perm [1,0,3,2]
+  x = dpp_add<0x4E>(x);   // quad_perm [2,3,0,1]
+  x = dpp_add<0x141>(x);  // row_half_mirror: the other quad of the 8-lane half row
+  if (TPR == 16) x = dpp_add<0x140>(x);  // row_mirror: the other half of the 16-lane row
   return x;
+}
+
+// acc + lo + hi of one packed bf16 pair (v_dot2c_f32_bf16 with a (1,1) operand): sums the ROUNDED values,
+// i.e. exactly what the MFMA consuming the packed operand sees.
+__device__ __forceinline__ float add_bf16_pair(uint32_t w, float acc) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  const bf2 one = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, w), one, acc, false);
 }
 
 __device__ __forceinline__ float sumsq8(u32x4 v) {
@@ -118,6 +135,18 @@ __device__ __forceinline__ bf16x8 pack_c_half(const f32x16& c, int s) {
   u32x4 w;
 #pragma unroll
   for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(c[8 * s + 2 * i], c[8 * s + 2 * i + 1]);
+  return as_bf16x8(w);
+}
+
+// same, and adds the eight packed values to `sum` (the scalar words are summed before the vector is
+// assembled: summing elements extracted back out of the assembled vector was miscompiled by hipcc 7.2)
+__device__ __forceinline__ bf16x8 pack_c_half_sum(const f32x16& c, int s, float& sum) {
+  const uint32_t w0 = pack_bf16x2(c[8 * s + 0], c[8 * s + 1]);
+  const uint32_t w1 = pack_bf16x2(c[8 * s + 2], c[8 * s + 3]);
+  const uint32_t w2 = pack_bf16x2(c[8 * s + 4], c[8 * s + 5]);
+  const uint32_t w3 = pack_bf16x2(c[8 * s + 6], c[8 * s + 7]);
+  sum = add_bf16_pair(w3, add_bf16_pair(w2, add_bf16_pair(w1, add_bf16_pair(w0, sum))));
+  const u32x4 w = {w0, w1, w2, w3};
   return as_bf16x8(w);
 }
 

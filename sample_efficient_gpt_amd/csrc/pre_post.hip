@@ -50,17 +50,29 @@ __global__ __launch_bounds__(256) void bwd_pre_kernel(KArgs a) {
   }
 }
 
-__global__ __launch_bounds__(256) void bwd_reduce_kernel(KArgs a) {
+constexpr int kReduceThreads = 1024;
+
+__global__ __launch_bounds__(kReduceThreads) void bwd_reduce_kernel(KArgs a) {
   const segpt_attn_params& p = a.p;
-  __shared__ float red[256];
+  __shared__ float red[kReduceThreads];
   __shared__ float tot[128];
   const int tid = threadIdx.x;
   const int D = p.D;
-  const int lanes = 256 / D;  // threads cooperating on one d (2, 4 or 8)
+  const int lanes = kReduceThreads / D;  // threads cooperating on one d
   const int d = tid % D, sl = tid / D;
-  float acc = 0.f;
-  for (int blk = sl; blk < a.n_dq_blocks; blk += lanes) acc += a.dg_part[(int64_t)blk * D + d];
-  red[tid] = acc;
+  // fixed summation order (deterministic); four independent chains hide the load latency
+  float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+  const float* src = a.dg_part + d;
+  const int n = a.n_dq_blocks;
+  int blk = sl;
+  for (; blk + 3 * lanes < n; blk += 4 * lanes) {
+    acc0 += src[(int64_t)blk * D];
+    acc1 += src[(int64_t)(blk + lanes) * D];
+    acc2 += src[(int64_t)(blk + 2 * lanes) * D];
+    acc3 += src[(int64_t)(blk + 3 * lanes) * D];
+  }
+  for (; blk < n; blk += lanes) acc0 += src[(int64_t)blk * D];
+  red[tid] = (acc0 + acc1) + (acc2 + acc3);
   __syncthreads();
   if (tid < D) {
     float t = 0.f;
@@ -99,15 +111,19 @@ __global__ __launch_bounds__(256) void bwd_reduce_kernel(KArgs a) {
   if (p.vr_coef) {
     __syncthreads();
     float s1 = 0.f, s2 = 0.f;
-    for (int blk = tid; blk < a.n_dkdv_blocks; blk += 256) {
-      s1 += a.dcoef_part[(int64_t)blk * 2];
-      s2 += a.dcoef_part[(int64_t)blk * 2 + 1];
+    for (int b2 = tid; b2 < a.n_dkdv_blocks; b2 += kReduceThreads) {
+      s1 += a.dcoef_part[(int64_t)b2 * 2];
+      s2 += a.dcoef_part[(int64_t)b2 * 2 + 1];
     }
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) { s1 += __shfl_xor(s1, o, 64); s2 += __shfl_xor(s2, o, 64); }
     if ((tid & 63) == 0) { red[(tid >> 6) * 2] = s1; red[(tid >> 6) * 2 + 1] = s2; }
     __syncthreads();
-    if (tid < 2) p.dvr_coef[tid] = red[tid] + red[2 + tid] + red[4 + tid] + red[6 + tid];
+    if (tid < 2) {
+      float t = 0.f;
+      for (int w = 0; w < kReduceThreads / 64; ++w) t += red[w * 2 + tid];
+      p.dvr_coef[tid] = t;
+    }
   }
 }
 
@@ -136,7 +152,7 @@ int launch_bwd_pre(const KArgs& a, hipStream_t st) {
 }
 
 int launch_bwd_reduce(const KArgs& a, hipStream_t st) {
-  hipLaunchKernelGGL(bwd_reduce_kernel, dim3(1), dim3(256), 0, st, a);
+  hipLaunchKernelGGL(bwd_reduce_kernel, dim3(1), dim3(kReduceThreads), 0, st, a);
   return (int)hipGetLastError();
 }
 

@@ -87,10 +87,13 @@ def compare(got, ref, dtype, names=None, label="", scales=None):
     `scales` overrides the magnitude the relative part refers to for the named outputs."""
     tol = TOL[dtype]
     errs = {}
+    failures = []
     for n in (names or ref.keys()):
         r = ref[n].double()
         g = got[n].double().reshape(r.shape)
-        assert torch.isfinite(g).all(), f"{label}{n}: non-finite values"
+        if not torch.isfinite(g).all():
+            failures.append(f"{label}{n}: non-finite values")
+            continue
         err = (g - r).abs()
         scale = r.abs().max() if n in REDUCED else r.abs()
         if scales and n in scales:
@@ -98,7 +101,8 @@ def compare(got, ref, dtype, names=None, label="", scales=None):
         bound = tol["atol"] + tol["rtol"] * scale
         errs[n] = float(err.max())
         bad = err > bound
-        assert not bad.any(), (
-            f"{label}{n}: {int(bad.sum())}/{bad.numel()} outside tolerance, max abs err {errs[n]:.3e} "
-            f"(ref max {float(r.abs().max()):.3e})")
+        if bad.any():
+            failures.append(f"{label}{n}: {int(bad.sum())}/{bad.numel()} outside tolerance, max abs err {errs[n]:.3e} "
+                            f"(ref max {float(r.abs().max()):.3e})")
+    assert not failures, "; ".join(failures)
     return errs
