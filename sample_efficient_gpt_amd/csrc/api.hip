@@ -23,7 +23,7 @@ size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 size_t elem_bytes(const segpt_attn_params& p) { return p.dtype == SEGPT_DTYPE_FP32 ? 4 : 2; }
 
 struct WsLayout {
-  size_t delta, do_eff, dg_part, dcoef_part, total;
+  size_t delta, do_eff, qhat, khat, vmix, dg_part, dcoef_part, total;
 };
 
 WsLayout bwd_layout(const segpt_attn_params& p) {
@@ -34,6 +34,15 @@ WsLayout bwd_layout(const segpt_attn_params& p) {
   off += align_up(rows * sizeof(float));
   w.do_eff = off;
   if (p.gate.ptr) off += align_up(rows * p.D * elem_bytes(p));
+  w.qhat = w.khat = w.vmix = off;
+  if (p.dtype == SEGPT_DTYPE_BF16) {
+    const size_t kvrows = (size_t)p.B * p.Hkv * p.Sk;
+    off += align_up(rows * p.D * 2);
+    w.khat = off;
+    off += align_up(kvrows * p.D * 2);
+    w.vmix = off;
+    if (p.v_first.ptr) off += align_up(kvrows * p.D * 2);
+  }
   w.dg_part = off;
   off += align_up((size_t)dq_blocks(p) * p.D * sizeof(float));
   w.dcoef_part = off;
@@ -159,6 +168,11 @@ static int bwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi
   a.do_eff = p->gate.ptr ? ws + w.do_eff : nullptr;
   a.dg_part = reinterpret_cast<float*>(ws + w.dg_part);
   a.dcoef_part = reinterpret_cast<float*>(ws + w.dcoef_part);
+  if (p->dtype == SEGPT_DTYPE_BF16) {
+    a.qhat = reinterpret_cast<uint16_t*>(ws + w.qhat);
+    a.khat = reinterpret_cast<uint16_t*>(ws + w.khat);
+    a.vmix = p->v_first.ptr ? reinterpret_cast<uint16_t*>(ws + w.vmix) : nullptr;
+  }
   a.n_dq_blocks = dq_blocks(*p);
   a.n_dkdv_blocks = dkdv_blocks(*p);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);

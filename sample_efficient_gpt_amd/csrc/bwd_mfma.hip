@@ -1,26 +1,29 @@
 // bf16 backward: two deterministic MFMA kernels (no floating-point atomics).
 //
-//  bwd_dq    query-stationary, same orientation as the forward:
-//              S^T  = Khat . Qhat^T          dP^T = V' . dO^T           (A from LDS row-major, B = registers)
-//              dS^T = P^T * (dP^T - delta)   T^T += Khat^T . dS^T       (A = transposing LDS read)
+// Operands are the normalised tensors written once by the backward pre-pass (pre_post.hip):
+//   Qhat = sm_scale*log2e * a_i q_i * g_q*g_k,  Khat = b_j k_j,  V' = c1 v + c2 v_first   (bf16).
+//
+//  bwd_dq    query-stationary, same orientation as the forward (a lane owns one query column):
+//              S^T  = Khat . Qhat^T - lse2        dP^T = V' . dO^T - delta     (A from LDS row-major,
+//              dS^T = exp2(S^T) * dP^T            T^T += Khat^T . dS^T          B = registers; the row
+//            statistics enter as the MFMA's C operand, so no subtraction is spent on them)
 //            epilogue: through the q normaliser, dq (bf16), and this workgroup's partial of the
 //            combined scale gradient dg[d] = sum_i sm_scale * (a_i q_id) * T_id.
-//  bwd_dkdv  key-stationary; a wave owns NKB blocks of 32 keys of one kv head and walks the query
-//            tiles of every query head of the group (dK/dV of a GQA group are summed in registers):
-//              S  = Qhat . Khat^T            dP = dO . V'^T             (A from LDS row-major, B = registers)
-//              dV'^T += dO^T . P             dKhat^T += Qhat^T . dS     (A = transposing LDS read)
+//  bwd_dkdv  key-stationary (a lane owns one key column); a wave owns 32 keys of one kv head and walks
+//            the query tiles of every query head of the group (dK/dV of a GQA group are summed in
+//            registers):
+//              S  = Qhat . Khat^T - lse2          dP = dO . V'^T - delta
+//              dV'^T += dO^T . P                  dKhat^T += Qhat^T . dS        (A = transposing LDS read)
 //            epilogue: through the k normaliser, dk, dv (= c1 dV'), dv_first (= c2 dV'), (dc1, dc2) partials.
 //
-// P is recomputed from the saved log-sum-exp: P = exp2(S2 - lse*log2e) with S2 in log2 units because
-// Qhat carries sm_scale*log2(e).  delta = rowsum(dO*O) comes from the bwd_pre kernel.
+// One workgroup = 4 waves (one per SIMD); several workgroups share a CU so that the softmax-like VALU
+// phase of one overlaps the MFMA phase of another.  Streamed tiles (64 rows) are double-buffered in LDS.
 #include "mfma_common.hpp"
 
 namespace segpt {
 namespace {
 
-template <int D> struct BwdCfg;
-template <> struct BwdCfg<64> { static constexpr int kNQB = 2, kNKB = 2; };
-template <> struct BwdCfg<128> { static constexpr int kNQB = 1, kNKB = 1; };
+constexpr int kBwdRows = 4 * 32;  // rows (queries for dQ, keys for dK/dV) owned by a workgroup
 
 __device__ __forceinline__ float gprod_at(const segpt_attn_params& p, int d) {
   float g = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
@@ -62,11 +65,55 @@ __device__ __forceinline__ void load_ct_block(const uint16_t* rowp, int mb, int 
   }
 }
 
-// ============================================================================================ dQ
-template <int D, int NQB, bool VR>
-__global__ __launch_bounds__(kThreadsM) void bwd_dq_bf16_kernel(KArgs a) {
+// ---- staging of two row-major bf16 tiles (64 rows x D) that need no arithmetic: global -> regs -> LDS
+template <int D>
+struct CopyRegs {
+  u32x4 a[Tile<D>::kPasses], b[Tile<D>::kPasses];
+};
+// rows r0.. of two tensors with the same (contiguous, stride D) layout starting at base pointers pa, pb
+template <int D>
+__device__ __forceinline__ void copy_load(const uint16_t* pa, int64_t stride_a, const uint16_t* pb, int64_t stride_b,
+                                          int row0, int nrows, CopyRegs<D>& r) {
   using T = Tile<D>;
-  constexpr int BQ = 4 * 32 * NQB;
+  const int tid = threadIdx.x;
+  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
+#pragma unroll
+  for (int ps = 0; ps < T::kPasses; ++ps) {
+    const int i = row0 + r0 + ps * T::kRowsPerPass;
+    if (i < nrows) {
+      r.a[ps] = *reinterpret_cast<const u32x4*>(pa + (int64_t)i * stride_a + chunk * 8);
+      r.b[ps] = *reinterpret_cast<const u32x4*>(pb + (int64_t)i * stride_b + chunk * 8);
+    } else {
+      r.a[ps] = u32x4{0, 0, 0, 0};
+      r.b[ps] = u32x4{0, 0, 0, 0};
+    }
+  }
+}
+template <int D>
+__device__ __forceinline__ void copy_store(const CopyRegs<D>& r, uint16_t* ta, uint16_t* tb) {
+  using T = Tile<D>;
+  const int tid = threadIdx.x;
+  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
+#pragma unroll
+  for (int ps = 0; ps < T::kPasses; ++ps) {
+    const int row = r0 + ps * T::kRowsPerPass;
+    *reinterpret_cast<u32x4*>(ta + row * T::kRS + chunk * 8) = r.a[ps];
+    *reinterpret_cast<u32x4*>(tb + row * T::kRS + chunk * 8) = r.b[ps];
+  }
+}
+
+__device__ __forceinline__ f32x16 splat16(float x) {
+  f32x16 v;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) v[r] = x;
+  return v;
+}
+
+// ============================================================================================ dQ
+template <int D>
+__global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel(KArgs a) {
+  using T = Tile<D>;
+  constexpr int BQ = kBwdRows;
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
   const segpt_attn_params& p = a.p;
@@ -80,59 +127,39 @@ __global__ __launch_bounds__(kThreadsM) void bwd_dq_bf16_kernel(KArgs a) {
   const WgCoord wg = decode_wg(blockIdx.x, n_qt, p.B, p.Hkv, rep);
   const int b = wg.b, g = wg.g, h = wg.g * rep + wg.hh;
   const int q0 = wg.tile * BQ;
-  const int qw0 = q0 + wave * 32 * NQB;
+  const int qw0 = q0 + wave * 32;
+  const int row_c = min(qw0 + ln, p.Sq - 1);  // this lane's query (clamped for the padding rows)
+  const int64_t ridx = ((int64_t)b * p.H + h) * p.Sq + row_c;
 
-  float c1 = 1.f, c2 = 0.f;
-  if (VR) { c1 = p.vr_coef[0]; c2 = p.vr_coef[1]; }
-
-  bf16x8 qreg[NQB][KS], doreg[NQB][KS];
-  float alpha[NQB], lse2[NQB], delta[NQB];
-#pragma unroll
-  for (int nb = 0; nb < NQB; ++nb) {
-    const int row = min(qw0 + 32 * nb + ln, p.Sq - 1);
-    const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row) + 8 * hh;
-    const uint16_t* dp = dout_row(a, b, h, row) + 8 * hh;
-    u32x4 raw[KS];
-    float ss = 0.f;
+  // stationary B operands: Qhat and dO rows of this lane's query
+  bf16x8 qreg[KS], doreg[KS];
+  {
+    const uint16_t* qp = a.qhat + ridx * D + 8 * hh;
+    const uint16_t* dp = dout_row(a, b, h, row_c) + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      raw[ks] = *reinterpret_cast<const u32x4*>(qp + 16 * ks);
-      doreg[nb][ks] = as_bf16x8(*reinterpret_cast<const u32x4*>(dp + 16 * ks));
-      ss += sumsq8(raw[ks]);
+      qreg[ks] = as_bf16x8(*reinterpret_cast<const u32x4*>(qp + 16 * ks));
+      doreg[ks] = as_bf16x8(*reinterpret_cast<const u32x4*>(dp + 16 * ks));
     }
-    ss = half_sum(ss);
-    alpha[nb] = fast_rsq(ss * (1.0f / D) + p.eps);
-    const float f = alpha[nb] * p.sm_scale * kLog2e;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      u32x4 w;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int d = 16 * ks + 8 * hh + 2 * i;
-        w[i] = pack_bf16x2(bf16lo(raw[ks][i]) * f * gprod_at(p, d), bf16hi(raw[ks][i]) * f * gprod_at(p, d + 1));
-      }
-      qreg[nb][ks] = as_bf16x8(w);
-    }
-    const int64_t ridx = ((int64_t)b * p.H + h) * p.Sq + row;
-    lse2[nb] = p.lse[ridx] * kLog2e;
-    delta[nb] = a.delta[ridx];
   }
+  // row statistics as MFMA C operands (every register of a lane belongs to the lane's query)
+  const f32x16 c_lse = splat16(-p.lse[ridx] * kLog2e);
+  const f32x16 c_del = splat16(-a.delta[ridx]);
 
-  f32x16 acc[MB][NQB];
+  f32x16 acc[MB];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < NQB; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = splat16(0.f);
 
   int kend = p.Sk;
   if (p.causal) kend = min(p.Sk, q0 + BQ + p.q_start);
   const int n_kt = (kend + kBK - 1) / kBK;
+  const uint16_t* kbase = a.khat + ((int64_t)b * p.Hkv + g) * p.Sk * D;
+  const uint16_t* vbase = a.vmix ? a.vmix + ((int64_t)b * p.Hkv + g) * p.Sk * D : row_ptr<uint16_t>(p.v, b, g, 0);
+  const int64_t vstride = a.vmix ? D : p.v.stride_s;
 
-  StageRegs<D> sr;
-  stage_load<D, VR>(p, b, g, 0, sr);
-  stage_store<D, VR>(sr, lds, lds + T::kElems, p.eps, c1, c2);
+  CopyRegs<D> sr;
+  copy_load<D>(kbase, D, vbase, vstride, 0, p.Sk, sr);
+  copy_store<D>(sr, lds, lds + T::kElems);
   __syncthreads();
 
   for (int jt = 0; jt < n_kt; ++jt) {
@@ -140,107 +167,82 @@ __global__ __launch_bounds__(kThreadsM) void bwd_dq_bf16_kernel(KArgs a) {
     const uint16_t* kt = lds + (jt & 1) * 2 * T::kElems;
     const uint16_t* vt = kt + T::kElems;
     const bool more = jt + 1 < n_kt;
-    if (more) stage_load<D, VR>(p, b, g, j0 + kBK, sr);
+    if (more) copy_load<D>(kbase, D, vbase, vstride, j0 + kBK, p.Sk, sr);
 
-    const bool active = !p.causal || j0 <= qw0 + 32 * NQB - 1 + p.q_start;
-    if (active) {
-      const bool need_mask = (p.causal && j0 + kBK - 1 > qw0 + p.q_start) || j0 + kBK > p.Sk;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        f32x16 s[NQB], dpv[NQB];
-#pragma unroll
-        for (int nb = 0; nb < NQB; ++nb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) { s[nb][r] = 0.f; dpv[nb][r] = 0.f; }
+    for (int kb = 0; kb < 2; ++kb) {
+      const int jb = j0 + 32 * kb;
+      const bool active = jb < p.Sk && (!p.causal || jb <= qw0 + 31 + p.q_start);  // wave-uniform
+      if (active) {
+        f32x16 s = c_lse, dpv = c_del;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8 kf = frag_rowmajor<D>(kt, kb, ks, lane);
-          const bf16x8 vf = frag_rowmajor<D>(vt, kb, ks, lane);
-#pragma unroll
-          for (int nb = 0; nb < NQB; ++nb) {
-            s[nb] = mfma32(kf, qreg[nb][ks], s[nb]);
-            dpv[nb] = mfma32(vf, doreg[nb][ks], dpv[nb]);
-          }
+          s = mfma32(frag_rowmajor<D>(kt, kb, ks, lane), qreg[ks], s);
+          dpv = mfma32(frag_rowmajor<D>(vt, kb, ks, lane), doreg[ks], dpv);
         }
-        bf16x8 dsb[2][NQB];
-#pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) {
-          const int qlim = p.causal ? min(qw0 + 32 * nb + ln + p.q_start, p.Sk - 1) : p.Sk - 1;
+        const bool need_mask = (p.causal && jb + 31 > qw0 + p.q_start) || jb + 32 > p.Sk;
+        if (need_mask) {
+          const int qlim = p.causal ? min(qw0 + ln + p.q_start, p.Sk - 1) : p.Sk - 1;
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            float pe = fast_exp2(s[nb][r] - lse2[nb]);
-            if (need_mask) {
-              const int key = j0 + 32 * kb + 8 * (r >> 2) + 4 * hh + (r & 3);
-              if (key > qlim) pe = 0.f;
-            }
-            s[nb][r] = pe * (dpv[nb][r] - delta[nb]);
+            const int key = jb + 8 * (r >> 2) + 4 * hh + (r & 3);
+            if (key > qlim) s[r] = -INFINITY;
           }
-          dsb[0][nb] = pack_c_half(s[nb], 0);
-          dsb[1][nb] = pack_c_half(s[nb], 1);
         }
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+        for (int r = 0; r < 16; ++r) s[r] = fast_exp2(s[r]) * dpv[r];
+        const bf16x8 ds0 = pack_c_half(s, 0), ds1 = pack_c_half(s, 1);
 #pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) {
-            const bf16x8 kT = frag_transposed<D>(kt, mb, 2 * kb + s2, lane);
-#pragma unroll
-            for (int nb = 0; nb < NQB; ++nb) acc[mb][nb] = mfma32(kT, dsb[s2][nb], acc[mb][nb]);
-          }
+        for (int mb = 0; mb < MB; ++mb) {
+          acc[mb] = mfma32(frag_transposed<D>(kt, mb, 2 * kb, lane), ds0, acc[mb]);
+          acc[mb] = mfma32(frag_transposed<D>(kt, mb, 2 * kb + 1, lane), ds1, acc[mb]);
+        }
       }
     }
     if (more) {
       uint16_t* nk = lds + ((jt + 1) & 1) * 2 * T::kElems;
-      stage_store<D, VR>(sr, nk, nk + T::kElems, p.eps, c1, c2);
+      copy_store<D>(sr, nk, nk + T::kElems);
     }
     __syncthreads();
   }
 
   // ---- epilogue.  acc = T^T: lane = query, registers = head-dim entries.
-  float dgl[MB][16];
+  const int row = qw0 + ln;
+  const bool live = row < p.Sq;
+  const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row_c);
+  float qv[MB][16];
+  float ss = 0.f;
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
+  for (int mb = 0; mb < MB; ++mb) {
+    load_ct_block(qp, mb, hh, qv[mb]);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) dgl[mb][r] = 0.f;
-#pragma unroll
-  for (int nb = 0; nb < NQB; ++nb) {
-    const int row = qw0 + 32 * nb + ln;
-    const bool live = row < p.Sq;
-    const int rc = live ? row : p.Sq - 1;
-    const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, rc);
-    float qv[MB][16], u[MB][16];
-    float dot = 0.f;
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      load_ct_block(qp, mb, hh, qv[mb]);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int d = 32 * mb + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const float t = acc[mb][nb][r] * p.sm_scale;
-        u[mb][r] = t * gprod_at(p, d);
-        dot += u[mb][r] * qv[mb][r];
-        if (live) dgl[mb][r] += t * alpha[nb] * qv[mb][r];
-      }
-    }
-    dot = half_sum(dot);
-    const float a3 = alpha[nb] * alpha[nb] * alpha[nb] * (1.0f / D) * dot;
-    uint16_t* op = row_ptr_mut<uint16_t>(p.dq, b, h, rc);
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      float val[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) val[r] = alpha[nb] * u[mb][r] - a3 * qv[mb][r];
-      store_ct_block(op, mb, hh, live, val);
-    }
+    for (int r = 0; r < 16; ++r) ss += qv[mb][r] * qv[mb][r];
   }
-  // workgroup partial of dg: column sums over the 128 (wave, lane%32) rows via LDS
+  ss = half_sum(ss);
+  const float alpha = fast_rsq(ss * (1.0f / D) + p.eps);
+  float dot = 0.f;
   float* red = reinterpret_cast<float*>(lds);
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int d = 32 * mb + 8 * (r >> 2) + 4 * hh + (r & 3);
-      red[(wave * 32 + ln) * (D + 1) + d] = dgl[mb][r];
+      const float t = acc[mb][r] * p.sm_scale;                 // sm_scale * T
+      red[(wave * 32 + ln) * (D + 1) + d] = live ? t * alpha * qv[mb][r] : 0.f;  // dg contribution of this row
+      acc[mb][r] = t * gprod_at(p, d);                         // u = dL/d(a q)
+      dot += acc[mb][r] * qv[mb][r];
     }
+  dot = half_sum(dot);
+  const float a3 = alpha * alpha * alpha * (1.0f / D) * dot;
+  uint16_t* op = row_ptr_mut<uint16_t>(p.dq, b, h, row_c);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    float val[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) val[r] = alpha * acc[mb][r] - a3 * qv[mb][r];
+    store_ct_block(op, mb, hh, live, val);
+  }
+  // workgroup partial of dg: column sums over the 128 (wave, lane%32) rows
   __syncthreads();
   if (tid < D) {
     float t = 0.f;
@@ -251,66 +253,14 @@ __global__ __launch_bounds__(kThreadsM) void bwd_dq_bf16_kernel(KArgs a) {
 
 // ============================================================================================ dK, dV
 template <int D>
-struct QStage {
-  u32x4 q[Tile<D>::kPasses], d[Tile<D>::kPasses];
-  float ld;  // lse*log2e (threads 0..63) or delta (threads 64..127)
-};
-
-template <int D>
-__device__ __forceinline__ void qstage_load(const KArgs& a, int b, int h, int i0, QStage<D>& r) {
+__global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kernel(KArgs a) {
   using T = Tile<D>;
-  const segpt_attn_params& p = a.p;
-  const int tid = threadIdx.x;
-  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
-#pragma unroll
-  for (int ps = 0; ps < T::kPasses; ++ps) {
-    const int i = i0 + r0 + ps * T::kRowsPerPass;
-    if (i < p.Sq) {
-      r.q[ps] = *reinterpret_cast<const u32x4*>(row_ptr<uint16_t>(p.q, b, h, i) + chunk * 8);
-      r.d[ps] = *reinterpret_cast<const u32x4*>(dout_row(a, b, h, i) + chunk * 8);
-    } else {
-      r.q[ps] = u32x4{0, 0, 0, 0};
-      r.d[ps] = u32x4{0, 0, 0, 0};
-    }
-  }
-  if (tid < 128) {
-    const int i = i0 + (tid & 63);
-    const int64_t ridx = ((int64_t)b * p.H + h) * p.Sq + min(i, p.Sq - 1);
-    if (tid < 64) r.ld = i < p.Sq ? p.lse[ridx] * kLog2e : INFINITY;  // +inf => P = 0 for padding rows
-    else r.ld = i < p.Sq ? a.delta[ridx] : 0.f;
-  }
-}
-
-template <int D>
-__device__ __forceinline__ void qstage_store(const QStage<D>& r, uint16_t* qt, uint16_t* dt, float* ldt, float eps,
-                                             float qscale, const float (&gch)[8]) {
-  using T = Tile<D>;
-  const int tid = threadIdx.x;
-  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
-#pragma unroll
-  for (int ps = 0; ps < T::kPasses; ++ps) {
-    const int row = r0 + ps * T::kRowsPerPass;
-    const float ss = row_group_sum<T::kTPR>(sumsq8(r.q[ps]));
-    const float f = fast_rsq(ss * (1.0f / D) + eps) * qscale;
-    u32x4 w;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      w[i] = pack_bf16x2(bf16lo(r.q[ps][i]) * f * gch[2 * i], bf16hi(r.q[ps][i]) * f * gch[2 * i + 1]);
-    *reinterpret_cast<u32x4*>(qt + row * T::kRS + chunk * 8) = w;
-    *reinterpret_cast<u32x4*>(dt + row * T::kRS + chunk * 8) = r.d[ps];
-  }
-  if (tid < 128) ldt[tid] = r.ld;  // [0,64): lse2, [64,128): delta
-}
-
-template <int D, int NKB, bool VR>
-__global__ __launch_bounds__(kThreadsM) void bwd_dkdv_bf16_kernel(KArgs a) {
-  using T = Tile<D>;
-  constexpr int BKV = 4 * 32 * NKB;
+  constexpr int BKV = kBwdRows;
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
   const segpt_attn_params& p = a.p;
   __shared__ __attribute__((aligned(16))) uint16_t lds[2 * 2 * T::kElems];
-  __shared__ __attribute__((aligned(16))) float ldl[2 * 128];
+  __shared__ __attribute__((aligned(16))) float ldl[2 * 128];  // per stage: [0,64) -lse2, [64,128) -delta
   __shared__ float red[8];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -321,54 +271,25 @@ __global__ __launch_bounds__(kThreadsM) void bwd_dkdv_bf16_kernel(KArgs a) {
   wg.tile = n_kvt - 1 - wg.tile;  // early key tiles see the most queries: issue them first
   const int b = wg.b, g = wg.g;
   const int k0 = wg.tile * BKV;
-  const int kw0 = k0 + wave * 32 * NKB;
+  const int kw0 = k0 + wave * 32;
+  const int key = kw0 + ln;
+  const int key_c = min(key, p.Sk - 1);
+  const int64_t kidx = ((int64_t)b * p.Hkv + g) * p.Sk + key_c;
 
-  float c1 = 1.f, c2 = 0.f;
-  if (VR) { c1 = p.vr_coef[0]; c2 = p.vr_coef[1]; }
-
-  // stationary operands: Khat and V' of this wave's keys, B-operand layout [nb][ks]
-  bf16x8 kreg[NKB][KS], vreg[NKB][KS];
-  float beta[NKB];
-#pragma unroll
-  for (int nb = 0; nb < NKB; ++nb) {
-    const int row = min(kw0 + 32 * nb + ln, p.Sk - 1);
-    const uint16_t* kp = row_ptr<uint16_t>(p.k, b, g, row) + 8 * hh;
-    const uint16_t* vp = row_ptr<uint16_t>(p.v, b, g, row) + 8 * hh;
-    u32x4 raw[KS];
-    float ss = 0.f;
+  // stationary B operands: Khat and V' rows of this lane's key
+  bf16x8 kreg[KS], vreg[KS];
+  {
+    const uint16_t* kp = a.khat + kidx * D + 8 * hh;
+    const uint16_t* vp = (a.vmix ? a.vmix + kidx * D : row_ptr<uint16_t>(p.v, b, g, key_c)) + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      raw[ks] = *reinterpret_cast<const u32x4*>(kp + 16 * ks);
-      ss += sumsq8(raw[ks]);
-      u32x4 vv = *reinterpret_cast<const u32x4*>(vp + 16 * ks);
-      if (VR) {
-        const u32x4 ff = *reinterpret_cast<const u32x4*>(row_ptr<uint16_t>(p.v_first, b, g, row) + 8 * hh + 16 * ks);
-        vv = mix8(vv, ff, c1, c2);
-      }
-      vreg[nb][ks] = as_bf16x8(vv);
+      kreg[ks] = as_bf16x8(*reinterpret_cast<const u32x4*>(kp + 16 * ks));
+      vreg[ks] = as_bf16x8(*reinterpret_cast<const u32x4*>(vp + 16 * ks));
     }
-    ss = half_sum(ss);
-    beta[nb] = fast_rsq(ss * (1.0f / D) + p.eps);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) kreg[nb][ks] = as_bf16x8(scale8(raw[ks], beta[nb]));
   }
-
-  f32x16 dvacc[MB][NKB], dkacc[MB][NKB];
+  f32x16 dvacc[MB], dkacc[MB];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < NKB; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { dvacc[mb][nb][r] = 0.f; dkacc[mb][nb][r] = 0.f; }
-
-  // per-thread slice of the scale product used when staging Qhat
-  float gch[8];
-  {
-    const int chunk = tid % T::kTPR;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) gch[e] = gprod_at(p, chunk * 8 + e);
-  }
-  const float qscale = p.sm_scale * kLog2e;
+  for (int mb = 0; mb < MB; ++mb) { dvacc[mb] = splat16(0.f); dkacc[mb] = splat16(0.f); }
 
   const int n_qt = (p.Sq + kBK - 1) / kBK;
   int qt_start = 0;
@@ -376,10 +297,30 @@ __global__ __launch_bounds__(kThreadsM) void bwd_dkdv_bf16_kernel(KArgs a) {
   const int n_vis = n_qt - qt_start;
   const int n_it = n_vis * rep;
 
-  QStage<D> qs;
+  // staging of one (head, query tile): Qhat and dO tiles plus the two row statistics
+  CopyRegs<D> sr;
+  float stat = 0.f;
+  auto stage_load_q = [&](int hq, int i0) {
+    const int h = g * rep + hq;
+    const int64_t base = ((int64_t)b * p.H + h) * p.Sq;
+    const uint16_t* dbase = a.do_eff ? reinterpret_cast<const uint16_t*>(a.do_eff) + base * D : row_ptr<uint16_t>(p.d_o, b, h, 0);
+    copy_load<D>(a.qhat + base * D, D, dbase, a.do_eff ? (int64_t)D : p.d_o.stride_s, i0, p.Sq, sr);
+    if (tid < 128) {
+      const int i = i0 + (tid & 63);
+      const int64_t ridx = base + min(i, p.Sq - 1);
+      if (tid < 64) stat = i < p.Sq ? -p.lse[ridx] * kLog2e : -INFINITY;  // -inf => P = 0 for padding rows
+      else stat = i < p.Sq ? -a.delta[ridx] : 0.f;
+    }
+  };
+  auto stage_store_q = [&](int stage) {
+    uint16_t* qt = lds + stage * 2 * T::kElems;
+    copy_store<D>(sr, qt, qt + T::kElems);
+    if (tid < 128) ldl[stage * 128 + tid] = stat;
+  };
+
   if (n_it > 0) {
-    qstage_load<D>(a, b, g * rep, qt_start * kBK, qs);
-    qstage_store<D>(qs, lds, lds + T::kElems, ldl, p.eps, qscale, gch);
+    stage_load_q(0, qt_start * kBK);
+    stage_store_q(0);
   }
   __syncthreads();
 
@@ -392,168 +333,139 @@ __global__ __launch_bounds__(kThreadsM) void bwd_dkdv_bf16_kernel(KArgs a) {
     const bool more = it + 1 < n_it;
     if (more) {
       const int hq2 = (it + 1) / n_vis;
-      const int i2 = (qt_start + (it + 1) - hq2 * n_vis) * kBK;
-      qstage_load<D>(a, b, g * rep + hq2, i2, qs);
+      stage_load_q(hq2, (qt_start + (it + 1) - hq2 * n_vis) * kBK);
     }
-    // wave-uniform: is any key of this wave visible to any query of the tile?
-    const bool active = !p.causal || kw0 <= i0 + kBK - 1 + p.q_start;
-    if (active) {
-      const bool need_mask = p.causal && kw0 + 32 * NKB - 1 > i0 + p.q_start;
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-        f32x16 s[NKB], dpv[NKB];
-#pragma unroll
-        for (int nb = 0; nb < NKB; ++nb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) { s[nb][r] = 0.f; dpv[nb][r] = 0.f; }
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8 qf = frag_rowmajor<D>(qt, qb, ks, lane);
-          const bf16x8 df = frag_rowmajor<D>(dt, qb, ks, lane);
-#pragma unroll
-          for (int nb = 0; nb < NKB; ++nb) {
-            s[nb] = mfma32(qf, kreg[nb][ks], s[nb]);
-            dpv[nb] = mfma32(df, vreg[nb][ks], dpv[nb]);
-          }
-        }
-        // row statistics of the 16 query rows this lane's registers map to
-        float lrow[16], drow[16];
+    for (int qb = 0; qb < 2; ++qb) {
+      const int ib = i0 + 32 * qb;  // first query of this 32-row block
+      // wave-uniform: is any key of this wave visible to any query of the block?
+      const bool active = ib < p.Sq && (!p.causal || kw0 <= ib + 31 + p.q_start);
+      if (active) {
+        // C operands: -lse2 / -delta of the 16 query rows this lane's registers map to
+        f32x16 s, dpv;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           const float4 l4 = *reinterpret_cast<const float4*>(lt + 32 * qb + 8 * c + 4 * hh);
           const float4 d4 = *reinterpret_cast<const float4*>(lt + 64 + 32 * qb + 8 * c + 4 * hh);
-          lrow[4 * c] = l4.x; lrow[4 * c + 1] = l4.y; lrow[4 * c + 2] = l4.z; lrow[4 * c + 3] = l4.w;
-          drow[4 * c] = d4.x; drow[4 * c + 1] = d4.y; drow[4 * c + 2] = d4.z; drow[4 * c + 3] = d4.w;
+          s[4 * c] = l4.x; s[4 * c + 1] = l4.y; s[4 * c + 2] = l4.z; s[4 * c + 3] = l4.w;
+          dpv[4 * c] = d4.x; dpv[4 * c + 1] = d4.y; dpv[4 * c + 2] = d4.z; dpv[4 * c + 3] = d4.w;
         }
-        bf16x8 pb[2][NKB], dsb[2][NKB];
 #pragma unroll
-        for (int nb = 0; nb < NKB; ++nb) {
-          const int key = kw0 + 32 * nb + ln;
+        for (int ks = 0; ks < KS; ++ks) {
+          s = mfma32(frag_rowmajor<D>(qt, qb, ks, lane), kreg[ks], s);
+          dpv = mfma32(frag_rowmajor<D>(dt, qb, ks, lane), vreg[ks], dpv);
+        }
+        const bool need_mask = p.causal && kw0 + 31 > ib + p.q_start;
+        if (need_mask) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            float pe = fast_exp2(s[nb][r] - lrow[r]);
-            if (need_mask) {
-              const int qi = i0 + 32 * qb + 8 * (r >> 2) + 4 * hh + (r & 3);
-              if (key > qi + p.q_start) pe = 0.f;
-            }
-            s[nb][r] = pe;
-            dpv[nb][r] = pe * (dpv[nb][r] - drow[r]);
+            const int qi = ib + 8 * (r >> 2) + 4 * hh + (r & 3);
+            if (key > qi + p.q_start) s[r] = -INFINITY;
           }
-          pb[0][nb] = pack_c_half(s[nb], 0);
-          pb[1][nb] = pack_c_half(s[nb], 1);
-          dsb[0][nb] = pack_c_half(dpv[nb], 0);
-          dsb[1][nb] = pack_c_half(dpv[nb], 1);
         }
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+        for (int r = 0; r < 16; ++r) {
+          s[r] = fast_exp2(s[r]);
+          dpv[r] *= s[r];
+        }
+        const bf16x8 p0 = pack_c_half(s, 0), p1 = pack_c_half(s, 1);
+        const bf16x8 ds0 = pack_c_half(dpv, 0), ds1 = pack_c_half(dpv, 1);
 #pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) {
-            const bf16x8 dT = frag_transposed<D>(dt, mb, 2 * qb + s2, lane);
-            const bf16x8 qT = frag_transposed<D>(qt, mb, 2 * qb + s2, lane);
-#pragma unroll
-            for (int nb = 0; nb < NKB; ++nb) {
-              dvacc[mb][nb] = mfma32(dT, pb[s2][nb], dvacc[mb][nb]);
-              dkacc[mb][nb] = mfma32(qT, dsb[s2][nb], dkacc[mb][nb]);
-            }
-          }
+        for (int mb = 0; mb < MB; ++mb) {
+          dvacc[mb] = mfma32(frag_transposed<D>(dt, mb, 2 * qb, lane), p0, dvacc[mb]);
+          dkacc[mb] = mfma32(frag_transposed<D>(qt, mb, 2 * qb, lane), ds0, dkacc[mb]);
+          dvacc[mb] = mfma32(frag_transposed<D>(dt, mb, 2 * qb + 1, lane), p1, dvacc[mb]);
+          dkacc[mb] = mfma32(frag_transposed<D>(qt, mb, 2 * qb + 1, lane), ds1, dkacc[mb]);
+        }
       }
     }
-    if (more) {
-      uint16_t* nq = lds + ((it + 1) & 1) * 2 * T::kElems;
-      qstage_store<D>(qs, nq, nq + T::kElems, ldl + ((it + 1) & 1) * 128, p.eps, qscale, gch);
-    }
+    if (more) stage_store_q((it + 1) & 1);
     __syncthreads();
   }
 
   // ---- epilogue: lane = key row, registers = head-dim entries
-  float s1 = 0.f, s2 = 0.f;
-#pragma unroll
-  for (int nb = 0; nb < NKB; ++nb) {
-    const int row = kw0 + 32 * nb + ln;
-    const bool live = row < p.Sk;
-    const int rc = live ? row : p.Sk - 1;
-    // dv, dv_first, (dc1, dc2)
-    uint16_t* ovp = row_ptr_mut<uint16_t>(p.dv, b, g, rc);
+  const bool live = key < p.Sk;
+  float c1 = 1.f, c2 = 0.f;
+  if (p.vr_coef) { c1 = p.vr_coef[0]; c2 = p.vr_coef[1]; }
+  {
+    uint16_t* ovp = row_ptr_mut<uint16_t>(p.dv, b, g, key_c);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       float val[16];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) val[r] = c1 * dvacc[mb][nb][r];
+      for (int r = 0; r < 16; ++r) val[r] = c1 * dvacc[mb][r];
       store_ct_block(ovp, mb, hh, live, val);
     }
-    if (VR) {
-      uint16_t* ofp = row_ptr_mut<uint16_t>(p.dv_first, b, g, rc);
-      const uint16_t* vp = row_ptr<uint16_t>(p.v, b, g, rc);
-      const uint16_t* fp = row_ptr<uint16_t>(p.v_first, b, g, rc);
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        float val[16], vv[16], ff[16];
-        load_ct_block(vp, mb, hh, vv);
-        load_ct_block(fp, mb, hh, ff);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          val[r] = c2 * dvacc[mb][nb][r];
-          if (live) { s1 += dvacc[mb][nb][r] * vv[r]; s2 += dvacc[mb][nb][r] * ff[r]; }
-        }
-        store_ct_block(ofp, mb, hh, live, val);
-      }
-    }
-    // dk through the normaliser: W = dL/dKhat (natural units), dk = b W - (b^3/D)(W.k) k
-    const uint16_t* kp = row_ptr<uint16_t>(p.k, b, g, rc);
-    float kv[MB][16];
-    float dot = 0.f;
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      load_ct_block(kp, mb, hh, kv[mb]);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dot += dkacc[mb][nb][r] * kv[mb][r];
-    }
-    dot = half_sum(dot) * kLn2;
-    const float b3 = beta[nb] * beta[nb] * beta[nb] * (1.0f / D) * dot;
-    uint16_t* okp = row_ptr_mut<uint16_t>(p.dk, b, g, rc);
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      float val[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) val[r] = beta[nb] * kLn2 * dkacc[mb][nb][r] - b3 * kv[mb][r];
-      store_ct_block(okp, mb, hh, live, val);
-    }
   }
-  if (VR) {
+  if (p.vr_coef) {
+    float s1 = 0.f, s2 = 0.f;
+    uint16_t* ofp = row_ptr_mut<uint16_t>(p.dv_first, b, g, key_c);
+    const uint16_t* vp = row_ptr<uint16_t>(p.v, b, g, key_c);
+    const uint16_t* fp = row_ptr<uint16_t>(p.v_first, b, g, key_c);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      float val[16], vv[16], ff[16];
+      load_ct_block(vp, mb, hh, vv);
+      load_ct_block(fp, mb, hh, ff);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        val[r] = c2 * dvacc[mb][r];
+        if (live) { s1 += dvacc[mb][r] * vv[r]; s2 += dvacc[mb][r] * ff[r]; }
+      }
+      store_ct_block(ofp, mb, hh, live, val);
+    }
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) { s1 += __shfl_xor(s1, o, 64); s2 += __shfl_xor(s2, o, 64); }
     if (lane == 0) { red[wave * 2] = s1; red[wave * 2 + 1] = s2; }
     __syncthreads();
     if (tid < 2) a.dcoef_part[(int64_t)blockIdx.x * 2 + tid] = red[tid] + red[2 + tid] + red[4 + tid] + red[6 + tid];
   }
+  // dk through the normaliser: W = ln2 * dkacc = dL/dKhat (natural units), dk = b W - (b^3/D)(W.k) k
+  {
+    const uint16_t* kp = row_ptr<uint16_t>(p.k, b, g, key_c);
+    float kv[MB][16];
+    float dot = 0.f, ss = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      load_ct_block(kp, mb, hh, kv[mb]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { dot += dkacc[mb][r] * kv[mb][r]; ss += kv[mb][r] * kv[mb][r]; }
+    }
+    dot = half_sum(dot) * kLn2;
+    ss = half_sum(ss);
+    const float beta = fast_rsq(ss * (1.0f / D) + p.eps);
+    const float b3 = beta * beta * beta * (1.0f / D) * dot;
+    uint16_t* okp = row_ptr_mut<uint16_t>(p.dk, b, g, key_c);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      float val[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) val[r] = beta * kLn2 * dkacc[mb][r] - b3 * kv[mb][r];
+      store_ct_block(okp, mb, hh, live, val);
+    }
+  }
 }
 
 template <int D>
 int launch_dkdv_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
-  constexpr int NKB = BwdCfg<D>::kNKB;
-  const int n_kvt = (p.Sk + 128 * NKB - 1) / (128 * NKB);
-  dim3 gk((unsigned)(n_kvt * p.Hkv * p.B)), block(kThreadsM);
-  if (p.v_first.ptr) hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D, NKB, true>), gk, block, 0, st, a);
-  else hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D, NKB, false>), gk, block, 0, st, a);
+  const int n_kvt = (p.Sk + kBwdRows - 1) / kBwdRows;
+  hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D>), dim3((unsigned)(n_kvt * p.Hkv * p.B)), dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 
 template <int D>
 int launch_dq_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
-  constexpr int NQB = BwdCfg<D>::kNQB;
-  const int n_qt = (p.Sq + 128 * NQB - 1) / (128 * NQB);
-  dim3 gq((unsigned)(n_qt * p.H * p.B)), block(kThreadsM);
-  if (p.v_first.ptr) hipLaunchKernelGGL((bwd_dq_bf16_kernel<D, NQB, true>), gq, block, 0, st, a);
-  else hipLaunchKernelGGL((bwd_dq_bf16_kernel<D, NQB, false>), gq, block, 0, st, a);
+  const int n_qt = (p.Sq + kBwdRows - 1) / kBwdRows;
+  hipLaunchKernelGGL((bwd_dq_bf16_kernel<D>), dim3((unsigned)(n_qt * p.H * p.B)), dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 
 }  // namespace
 
-int bf16_dq_rows_per_block(int D) { return D == 64 ? 128 * BwdCfg<64>::kNQB : 128 * BwdCfg<128>::kNQB; }
-int bf16_dkdv_rows_per_block(int D) { return D == 64 ? 128 * BwdCfg<64>::kNKB : 128 * BwdCfg<128>::kNKB; }
+int bf16_dq_rows_per_block(int) { return kBwdRows; }
+int bf16_dkdv_rows_per_block(int) { return kBwdRows; }
 
 int launch_bwd_dkdv_bf16(const KArgs& a, hipStream_t st) {
   if (a.p.D == 64) return launch_dkdv_t<64>(a, st);

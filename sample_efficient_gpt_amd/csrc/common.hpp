@@ -16,6 +16,9 @@ struct KArgs {
   segpt_attn_params p;
   float* delta;       // [B,H,Sq] fp32: rowsum(dO_eff * o)
   void* do_eff;       // [B,H,Sq,D] dtype, contiguous: gate-scaled dO (only when gated)
+  uint16_t* qhat;     // [B,H,Sq,D]   bf16: sm_scale*log2e * a_i q_i * g_q*g_k   (bf16 path only)
+  uint16_t* khat;     // [B,Hkv,Sk,D] bf16: b_j k_j                               (bf16 path only)
+  uint16_t* vmix;     // [B,Hkv,Sk,D] bf16: c1 v + c2 v_first (only with a value residual, else NULL)
   float* dg_part;     // [n_dq_blocks, D] fp32 partial sums of the combined scale gradient
   float* dcoef_part;  // [n_dkdv_blocks, 2] fp32 partial sums of (dc1, dc2)
   int32_t n_dq_blocks;

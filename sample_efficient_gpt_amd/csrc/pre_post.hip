@@ -1,5 +1,7 @@
 // HBM-bound helper kernels of the backward:
-//   bwd_pre     delta_i = rowsum(dY_i * Y_i); with a gate also dgate = (1 - sigmoid(z)) * delta and
+//   bwd_pre     delta_i = rowsum(dY_i * Y_i); on the bf16 path also the normalised operands Qhat, Khat and
+//               V' that the two MFMA kernels stream (so their inner loops carry no norm arithmetic);
+//               with a gate also dgate = (1 - sigmoid(z)) * delta and
 //               dO_eff = gate_scale * sigmoid(z) * dY  (Y is the saved, already gated output, so
 //               rowsum(dO_eff * O) == rowsum(dY * Y) and no division by the gate is needed).
 //   bwd_reduce  second stage of the scale-gradient reduction: sums the per-workgroup partial
@@ -33,6 +35,25 @@ __global__ __launch_bounds__(256) void bwd_pre_kernel(KArgs a) {
   for (int e = 0; e < V; ++e) acc += y[e] * dy[e];
 #pragma unroll
   for (int o = 1; o < TPR; o <<= 1) acc += __shfl_xor(acc, o, 64);
+  if (a.qhat) {  // bf16 path: the normalised, scaled query row the two MFMA kernels consume
+    float q[V];
+    Elem<T>::load(row_ptr<T>(p.q, b, h, s) + part * V, q);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < V; ++e) ss += q[e] * q[e];
+#pragma unroll
+    for (int o = 1; o < TPR; o <<= 1) ss += __shfl_xor(ss, o, 64);
+    const float f = (1.0f / sqrtf(ss * (1.0f / D) + p.eps)) * p.sm_scale * kLog2e;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const int d = part * V + e;
+      float g = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
+      if (p.gk_numel == 1) g *= p.g_k[0];
+      else if (p.gk_numel > 1) g *= p.g_k[d];
+      q[e] *= f * g;
+    }
+    if (live) Elem<T>::store(reinterpret_cast<T*>(a.qhat) + r * D + part * V, q);
+  }
   if (!live) return;
   if (part == 0) a.delta[r] = acc;
   if (p.gate.ptr) {
@@ -47,6 +68,43 @@ __global__ __launch_bounds__(256) void bwd_pre_kernel(KArgs a) {
 #pragma unroll
     for (int e = 0; e < V; ++e) dy[e] *= f;
     Elem<T>::store(reinterpret_cast<T*>(a.do_eff) + r * D + part * V, dy);
+  }
+}
+
+// bf16 path: Khat = b_j k_j and (with a value residual) V' = c1 v + c2 v_first, one row per 8/16 lanes
+template <int D>
+__global__ __launch_bounds__(256) void bwd_prep_kv_kernel(KArgs a) {
+  const segpt_attn_params& p = a.p;
+  constexpr int TPR = D / 8;
+  constexpr int RPB = 256 / TPR;
+  const int tid = threadIdx.x;
+  const int part = tid % TPR;
+  const int64_t rid = (int64_t)blockIdx.x * RPB + tid / TPR;  // flat (b, g, s)
+  const int64_t nrows = (int64_t)p.B * p.Hkv * p.Sk;
+  const bool live = rid < nrows;
+  const int64_t r = live ? rid : nrows - 1;
+  const int s = (int)(r % p.Sk);
+  const int g = (int)((r / p.Sk) % p.Hkv);
+  const int b = (int)(r / ((int64_t)p.Sk * p.Hkv));
+  float k[8];
+  Elem<uint16_t>::load(row_ptr<uint16_t>(p.k, b, g, s) + part * 8, k);
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ss += k[e] * k[e];
+#pragma unroll
+  for (int o = 1; o < TPR; o <<= 1) ss += __shfl_xor(ss, o, 64);
+  const float beta = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) k[e] *= beta;
+  if (live) Elem<uint16_t>::store(a.khat + r * D + part * 8, k);
+  if (a.vmix) {
+    const float c1 = p.vr_coef[0], c2 = p.vr_coef[1];
+    float v[8], f[8];
+    Elem<uint16_t>::load(row_ptr<uint16_t>(p.v, b, g, s) + part * 8, v);
+    Elem<uint16_t>::load(row_ptr<uint16_t>(p.v_first, b, g, s) + part * 8, f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = c1 * v[e] + c2 * f[e];
+    if (live) Elem<uint16_t>::store(a.vmix + r * D + part * 8, v);
   }
 }
 
@@ -148,7 +206,16 @@ int launch_pre_t(const KArgs& a, hipStream_t st) {
 }  // namespace
 
 int launch_bwd_pre(const KArgs& a, hipStream_t st) {
-  return a.p.dtype == SEGPT_DTYPE_FP32 ? launch_pre_t<float>(a, st) : launch_pre_t<uint16_t>(a, st);
+  if (a.p.dtype == SEGPT_DTYPE_FP32) return launch_pre_t<float>(a, st);
+  int rc = launch_pre_t<uint16_t>(a, st);
+  if (rc) return rc;
+  const segpt_attn_params& p = a.p;
+  const int64_t nrows = (int64_t)p.B * p.Hkv * p.Sk;
+  const int rpb = 256 / (p.D / 8);
+  dim3 grid((unsigned)((nrows + rpb - 1) / rpb)), block(256);
+  if (p.D == 64) hipLaunchKernelGGL(bwd_prep_kv_kernel<64>, grid, block, 0, st, a);
+  else hipLaunchKernelGGL(bwd_prep_kv_kernel<128>, grid, block, 0, st, a);
+  return (int)hipGetLastError();
 }
 
 int launch_bwd_reduce(const KArgs& a, hipStream_t st) {
