@@ -87,7 +87,7 @@ def main():
     torch.cuda.set_device(dev)
     x = make_inputs(c, device=dev)
     plan = AttnPlan(x, eps=c.eps, sm_scale=c.sm_scale, gate_scale=c.gate_scale, backward=c.backward)
-    names = ["fwd"] + (["bwd_pre", "bwd_dkdv", "bwd_dq", "bwd_reduce"] if c.backward else [])
+    names = ["fwd"] + (["bwd_pre", "bwd_dq", "bwd_dkdv", "bwd_reduce"] if c.backward else [])
 
     def step(events=None):
         if events is not None:
@@ -131,7 +131,8 @@ def main():
     achieved = credited[dom] / (kern_ms[dom] * 1e-3) / 1e12
     elem = 2
     hbm_bytes = {  # algorithmic bytes of the HBM-bound helpers
-        "bwd_pre": c.B * c.H * c.S * (2 * c.D * elem + 4) + (c.B * c.H * c.S * (c.D * elem + 2 * elem) if c.extras else 0),
+        # K in, Khat out (+ v, v_first in, V' out with a value residual)
+        "bwd_pre": c.B * c.Hkv * c.S * c.D * elem * (5 if c.extras else 2),
     }
     kernels = {}
     for n in names:

@@ -58,11 +58,13 @@ extern "C" {
 #define SEGPT_E_ALIGN -10      /* a base pointer is not 16-byte aligned                     */
 #define SEGPT_E_STAGE -11      /* unknown stage passed to segpt_attn_bwd_stage              */
 
-/* the four launches segpt_attn_bwd() makes, in this order */
-#define SEGPT_BWD_STAGE_PRE 0    /* delta = rowsum(dY*Y); gate: dgate and the gate-scaled dO      */
-#define SEGPT_BWD_STAGE_DKDV 1   /* dK, dV (, dV_first, partial sums of d vr_coef)                */
-#define SEGPT_BWD_STAGE_DQ 2     /* dQ and the per-workgroup partials of the scale gradient       */
-#define SEGPT_BWD_STAGE_REDUCE 3 /* dg_q, dg_k, d vr_coef from the partials                       */
+/* the four stages segpt_attn_bwd() runs, in this order */
+#define SEGPT_BWD_STAGE_PRE 0    /* bf16: normalised Khat (and V' = c1 v + c2 v_first) into the workspace;
+                                    fp32: delta = rowsum(dY*Y), dgate and the gate-scaled dO            */
+#define SEGPT_BWD_STAGE_DQ 1     /* dQ and the per-workgroup partials of the scale gradient; on the bf16
+                                    path also delta, dgate, Qhat and the gate-scaled dO for stage 2      */
+#define SEGPT_BWD_STAGE_DKDV 2   /* dK, dV (, dV_first, partial sums of d vr_coef)                       */
+#define SEGPT_BWD_STAGE_REDUCE 3 /* dg_q, dg_k, d vr_coef from the partials                              */
 
 /* [B, heads, S, D] tensor view; the D axis is contiguous (stride 1). Strides in ELEMENTS.
  * The reference's `(h b) S D` flatten (attention.py:199) is stride_b = S*D, stride_h = B*S*D;
@@ -141,7 +143,7 @@ int segpt_attn_bwd(const segpt_attn_params* p, void* stream);
 
 /* One launch of the backward, for profilers and benchmarks that time the kernels separately:
  * segpt_attn_bwd(p, s) is exactly stages 0, 1, 2, 3 in this order on one stream with the same params
- * and workspace.  Stage 0 must have run before 1 and 2, and 2 before 3.  No counterpart in the
+ * and workspace.  Each stage needs the earlier ones to have run on the same workspace.  No counterpart in the
  * reference (its backward is the single kernel triton_flash_attn_qknorm.py:125-255). */
 int segpt_attn_bwd_stage(const segpt_attn_params* p, int stage, void* stream);
 

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libsegpt_attn.so")
 SEGPT_ABI_VERSION = 1
 SEGPT_DTYPE_BF16 = 0
 SEGPT_DTYPE_FP32 = 1
-BWD_STAGES = ("pre", "dkdv", "dq", "reduce")  # SEGPT_BWD_STAGE_* = index
+BWD_STAGES = ("pre", "dq", "dkdv", "reduce")  # SEGPT_BWD_STAGE_* = index
 
 EXPORTED_SYMBOLS = (
     "segpt_abi_version",

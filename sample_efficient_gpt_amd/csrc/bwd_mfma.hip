@@ -1,7 +1,9 @@
 // bf16 backward: two deterministic MFMA kernels (no floating-point atomics).
 //
-// Operands are the normalised tensors written once by the backward pre-pass (pre_post.hip):
-//   Qhat = sm_scale*log2e * a_i q_i * g_q*g_k,  Khat = b_j k_j,  V' = c1 v + c2 v_first   (bf16).
+// Operands are normalised tensors held in the workspace (bf16):
+//   Khat = b_j k_j and V' = c1 v + c2 v_first, written by the key/value pre-pass (pre_post.hip);
+//   Qhat = sm_scale*log2e * a_i q_i * g_q*g_k, delta and the gate-scaled dO, written by the dQ kernel's
+//   prologue for the dK/dV kernel that runs after it.
 //
 //  bwd_dq    query-stationary, same orientation as the forward (a lane owns one query column):
 //              S^T  = Khat . Qhat^T - lse2        dP^T = V' . dO^T - delta     (A from LDS row-major,
@@ -30,12 +32,6 @@ __device__ __forceinline__ float gprod_at(const segpt_attn_params& p, int d) {
   if (p.gk_numel == 1) g *= p.g_k[0];
   else if (p.gk_numel > 1) g *= p.g_k[d];
   return g;
-}
-
-__device__ __forceinline__ const uint16_t* dout_row(const KArgs& a, int b, int h, int s) {
-  const segpt_attn_params& p = a.p;
-  if (a.do_eff) return reinterpret_cast<const uint16_t*>(a.do_eff) + (((int64_t)b * p.H + h) * p.Sq + s) * p.D;
-  return row_ptr<uint16_t>(p.d_o, b, h, s);
 }
 
 // store a C tile column block: lane = row of the output tensor, registers = 32 consecutive columns
@@ -109,7 +105,19 @@ __device__ __forceinline__ f32x16 splat16(float x) {
   return v;
 }
 
+constexpr int kStages = 3;  // LDS ring of streamed tiles: tile t lives in stage t % 3
+
 // ============================================================================================ dQ
+// Also the producer of the per-query-row quantities the dK/dV kernel streams afterwards: Qhat, delta
+// and (with a gate) the gate-scaled dO and dgate.
+//
+// Software pipeline over 32-key blocks n (two per staged tile), one barrier per tile:
+//   B(n)  S^T, dP^T MFMAs from the row-major fragments requested one block earlier
+//   C(n)  request the transposed Khat fragments of block n
+//   D(n)  dS^T = exp2(S^T) * dP^T, pack to bf16
+//   A(n+1) request the row-major fragments of block n+1 (possibly the next tile, already in LDS)
+//   E(n)  T^T += Khat^T dS^T MFMAs
+// Tiles are stored two tiles ahead of their use so that A(n+1) never waits for a barrier.
 template <int D>
 __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel(KArgs a) {
   using T = Tile<D>;
@@ -117,8 +125,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
   const segpt_attn_params& p = a.p;
-  __shared__ __attribute__((aligned(16))) uint16_t lds[2 * 2 * T::kElems];
-  static_assert(2 * 2 * T::kElems * 2 >= 128 * (D + 1) * 4, "LDS reuse for the dg partial");
+  __shared__ __attribute__((aligned(16))) uint16_t lds[kStages * 2 * T::kElems];
+  static_assert(kStages * 2 * T::kElems * 2 >= 128 * (D + 1) * 4, "LDS reuse for the dg partial");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, hh = lane >> 5;
@@ -128,27 +136,10 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   const int b = wg.b, g = wg.g, h = wg.g * rep + wg.hh;
   const int q0 = wg.tile * BQ;
   const int qw0 = q0 + wave * 32;
-  const int row_c = min(qw0 + ln, p.Sq - 1);  // this lane's query (clamped for the padding rows)
+  const int row = qw0 + ln;
+  const bool live = row < p.Sq;
+  const int row_c = live ? row : p.Sq - 1;  // padding lanes recompute the last row and store nothing
   const int64_t ridx = ((int64_t)b * p.H + h) * p.Sq + row_c;
-
-  // stationary B operands: Qhat and dO rows of this lane's query
-  bf16x8 qreg[KS], doreg[KS];
-  {
-    const uint16_t* qp = a.qhat + ridx * D + 8 * hh;
-    const uint16_t* dp = dout_row(a, b, h, row_c) + 8 * hh;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      qreg[ks] = as_bf16x8(*reinterpret_cast<const u32x4*>(qp + 16 * ks));
-      doreg[ks] = as_bf16x8(*reinterpret_cast<const u32x4*>(dp + 16 * ks));
-    }
-  }
-  // row statistics as MFMA C operands (every register of a lane belongs to the lane's query)
-  const f32x16 c_lse = splat16(-p.lse[ridx] * kLog2e);
-  const f32x16 c_del = splat16(-a.delta[ridx]);
-
-  f32x16 acc[MB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) acc[mb] = splat16(0.f);
 
   int kend = p.Sk;
   if (p.causal) kend = min(p.Sk, q0 + BQ + p.q_start);
@@ -157,73 +148,146 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   const uint16_t* vbase = a.vmix ? a.vmix + ((int64_t)b * p.Hkv + g) * p.Sk * D : row_ptr<uint16_t>(p.v, b, g, 0);
   const int64_t vstride = a.vmix ? D : p.v.stride_s;
 
+  // ---- first two tiles on their way to LDS while the query-row prologue runs
   CopyRegs<D> sr;
   copy_load<D>(kbase, D, vbase, vstride, 0, p.Sk, sr);
   copy_store<D>(sr, lds, lds + T::kElems);
-  __syncthreads();
+  if (n_kt > 1) {
+    copy_load<D>(kbase, D, vbase, vstride, kBK, p.Sk, sr);
+    copy_store<D>(sr, lds + 2 * T::kElems, lds + 3 * T::kElems);
+  }
 
-  for (int jt = 0; jt < n_kt; ++jt) {
-    const int j0 = jt * kBK;
-    const uint16_t* kt = lds + (jt & 1) * 2 * T::kElems;
-    const uint16_t* vt = kt + T::kElems;
-    const bool more = jt + 1 < n_kt;
-    if (more) copy_load<D>(kbase, D, vbase, vstride, j0 + kBK, p.Sk, sr);
-
+  // ---- query-row prologue: alpha, Qhat, delta, gate; B operands stay in registers
+  bf16x8 qreg[KS], doreg[KS];
+  float alpha, delta;
+  {
+    const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row_c) + 8 * hh;
+    const uint16_t* yp = row_ptr<uint16_t>(p.o, b, h, row_c) + 8 * hh;
+    const uint16_t* dp = row_ptr<uint16_t>(p.d_o, b, h, row_c) + 8 * hh;
+    u32x4 qraw[KS], dyraw[KS];
+    float ss = 0.f, dl = 0.f;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const int jb = j0 + 32 * kb;
-      const bool active = jb < p.Sk && (!p.causal || jb <= qw0 + 31 + p.q_start);  // wave-uniform
-      if (active) {
-        f32x16 s = c_lse, dpv = c_del;
+    for (int ks = 0; ks < KS; ++ks) {
+      qraw[ks] = *reinterpret_cast<const u32x4*>(qp + 16 * ks);
+      dyraw[ks] = *reinterpret_cast<const u32x4*>(dp + 16 * ks);
+      const u32x4 y = *reinterpret_cast<const u32x4*>(yp + 16 * ks);
+      ss += sumsq8(qraw[ks]);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          s = mfma32(frag_rowmajor<D>(kt, kb, ks, lane), qreg[ks], s);
-          dpv = mfma32(frag_rowmajor<D>(vt, kb, ks, lane), doreg[ks], dpv);
-        }
-        const bool need_mask = (p.causal && jb + 31 > qw0 + p.q_start) || jb + 32 > p.Sk;
-        if (need_mask) {
-          const int qlim = p.causal ? min(qw0 + ln + p.q_start, p.Sk - 1) : p.Sk - 1;
+      for (int i = 0; i < 4; ++i) dl += bf16lo(y[i]) * bf16lo(dyraw[ks][i]) + bf16hi(y[i]) * bf16hi(dyraw[ks][i]);
+    }
+    ss = half_sum(ss);
+    delta = half_sum(dl);
+    alpha = fast_rsq(ss * (1.0f / D) + p.eps);
+    const float f = alpha * p.sm_scale * kLog2e;
+    float gfac = 1.f;
+    if (p.gate.ptr) {
+      const float z = bf16_to_f32(reinterpret_cast<const uint16_t*>(p.gate.ptr)[(int64_t)b * p.gate.stride_b + (int64_t)row_c * p.gate.stride_s + (int64_t)h * p.gate.stride_h]);
+      const float sg = 1.0f / (1.0f + __expf(-z));
+      gfac = p.gate_scale * sg;
+      if (live && hh == 0)
+        reinterpret_cast<uint16_t*>(p.dgate.ptr)[(int64_t)b * p.dgate.stride_b + (int64_t)row * p.dgate.stride_s + (int64_t)h * p.dgate.stride_h] = f32_to_bf16((1.0f - sg) * delta);
+    }
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = jb + 8 * (r >> 2) + 4 * hh + (r & 3);
-            if (key > qlim) s[r] = -INFINITY;
-          }
-        }
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4 w;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = fast_exp2(s[r]) * dpv[r];
-        const bf16x8 ds0 = pack_c_half(s, 0), ds1 = pack_c_half(s, 1);
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-          acc[mb] = mfma32(frag_transposed<D>(kt, mb, 2 * kb, lane), ds0, acc[mb]);
-          acc[mb] = mfma32(frag_transposed<D>(kt, mb, 2 * kb + 1, lane), ds1, acc[mb]);
-        }
+      for (int i = 0; i < 4; ++i) {
+        const int d = 16 * ks + 8 * hh + 2 * i;
+        w[i] = pack_bf16x2(bf16lo(qraw[ks][i]) * f * gprod_at(p, d), bf16hi(qraw[ks][i]) * f * gprod_at(p, d + 1));
+      }
+      qreg[ks] = as_bf16x8(w);
+      if (live) *reinterpret_cast<u32x4*>(a.qhat + ridx * D + 16 * ks + 8 * hh) = w;
+      if (p.gate.ptr) {
+        const u32x4 e = scale8(dyraw[ks], gfac);
+        doreg[ks] = as_bf16x8(e);
+        if (live) *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(a.do_eff) + ridx * D + 16 * ks + 8 * hh) = e;
+      } else {
+        doreg[ks] = as_bf16x8(dyraw[ks]);
       }
     }
-    if (more) {
-      uint16_t* nk = lds + ((jt + 1) & 1) * 2 * T::kElems;
+    if (live && hh == 0) a.delta[ridx] = delta;
+  }
+  // row statistics as MFMA C operands (every register of a lane belongs to the lane's query)
+  const f32x16 c_lse = splat16(-p.lse[ridx] * kLog2e);
+  const f32x16 c_del = splat16(-delta);
+
+  f32x16 acc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = splat16(0.f);
+
+  // blocks this wave has to visit (causal: up to the block holding its last query's diagonal)
+  int n_act = (min(kend, p.Sk) + 31) / 32;
+  if (p.causal) n_act = min(n_act, (qw0 + 31 + p.q_start) / 32 + 1);
+  const int qlim = p.causal ? min(row + p.q_start, p.Sk - 1) : p.Sk - 1;  // last visible key of this lane's query
+
+  bf16x8 kf[KS], vf[KS];
+  auto request_rowmajor = [&](int blk) {
+    const uint16_t* kt = lds + ((blk >> 1) % kStages) * 2 * T::kElems;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      kf[ks] = frag_rowmajor<D>(kt, blk & 1, ks, lane);
+      vf[ks] = frag_rowmajor<D>(kt + T::kElems, blk & 1, ks, lane);
+    }
+  };
+  auto step = [&](int blk) {
+    const uint16_t* kt = lds + ((blk >> 1) % kStages) * 2 * T::kElems;
+    const int kb = blk & 1;
+    const int jb = blk * 32;
+    f32x16 s = c_lse, dpv = c_del;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      s = mfma32(kf[ks], qreg[ks], s);
+      dpv = mfma32(vf[ks], doreg[ks], dpv);
+    }
+    bf16x8 kT[MB][2];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      kT[mb][0] = frag_transposed<D>(kt, mb, 2 * kb, lane);
+      kT[mb][1] = frag_transposed<D>(kt, mb, 2 * kb + 1, lane);
+    }
+    if ((p.causal && jb + 31 > qw0 + p.q_start) || jb + 32 > p.Sk) {  // block touches the diagonal or the end of the keys
+      // register r holds key jb + 4hh + c_r, c_r = 8(r/4) + r%4: masked iff c_r > qlim - jb - 4hh
+      const int t = qlim - jb - 4 * hh;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (8 * (r >> 2) + (r & 3) > t) s[r] = -INFINITY;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = fast_exp2(s[r]) * dpv[r];
+    const bf16x8 ds0 = pack_c_half(s, 0), ds1 = pack_c_half(s, 1);
+    if (blk + 1 < n_act) request_rowmajor(blk + 1);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      acc[mb] = mfma32(kT[mb][0], ds0, acc[mb]);
+      acc[mb] = mfma32(kT[mb][1], ds1, acc[mb]);
+    }
+  };
+
+  // The loads left in flight across the loop must be the YOUNGEST vector-memory operations: every wait
+  // for an older load (the row prologue above) would otherwise also drain them in each iteration.
+  drain_vector_loads();
+  if (n_kt > 2) copy_load<D>(kbase, D, vbase, vstride, 2 * kBK, p.Sk, sr);
+  __syncthreads();
+  if (n_act > 0) request_rowmajor(0);
+  for (int jt = 0; jt < n_kt; ++jt) {
+    if (2 * jt < n_act) step(2 * jt);
+    if (2 * jt + 1 < n_act) step(2 * jt + 1);
+    if (jt + 2 < n_kt) {
+      uint16_t* nk = lds + ((jt + 2) % kStages) * 2 * T::kElems;
       copy_store<D>(sr, nk, nk + T::kElems);
+      if (jt + 3 < n_kt) copy_load<D>(kbase, D, vbase, vstride, (jt + 3) * kBK, p.Sk, sr);
     }
     __syncthreads();
   }
 
   // ---- epilogue.  acc = T^T: lane = query, registers = head-dim entries.
-  const int row = qw0 + ln;
-  const bool live = row < p.Sq;
   const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row_c);
+  float dot = 0.f;
+  float* red = reinterpret_cast<float*>(lds);
   float qv[MB][16];
-  float ss = 0.f;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     load_ct_block(qp, mb, hh, qv[mb]);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) ss += qv[mb][r] * qv[mb][r];
-  }
-  ss = half_sum(ss);
-  const float alpha = fast_rsq(ss * (1.0f / D) + p.eps);
-  float dot = 0.f;
-  float* red = reinterpret_cast<float*>(lds);
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int d = 32 * mb + 8 * (r >> 2) + 4 * hh + (r & 3);
@@ -232,6 +296,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
       acc[mb][r] = t * gprod_at(p, d);                         // u = dL/d(a q)
       dot += acc[mb][r] * qv[mb][r];
     }
+  }
   dot = half_sum(dot);
   const float a3 = alpha * alpha * alpha * (1.0f / D) * dot;
   uint16_t* op = row_ptr_mut<uint16_t>(p.dq, b, h, row_c);
@@ -252,6 +317,9 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
 }
 
 // ============================================================================================ dK, dV
+// Same pipeline with the roles swapped: the streamed tiles are Qhat / dO (64 queries of one head), the
+// blocks are 32 queries, and B(n) starts from the two row statistics of the block, read from LDS
+// straight into the accumulators of S and dP.
 template <int D>
 __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kernel(KArgs a) {
   using T = Tile<D>;
@@ -259,8 +327,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
   const segpt_attn_params& p = a.p;
-  __shared__ __attribute__((aligned(16))) uint16_t lds[2 * 2 * T::kElems];
-  __shared__ __attribute__((aligned(16))) float ldl[2 * 128];  // per stage: [0,64) -lse2, [64,128) -delta
+  __shared__ __attribute__((aligned(16))) uint16_t lds[kStages * 2 * T::kElems];
+  __shared__ __attribute__((aligned(16))) float ldl[kStages * 128];  // per stage: [0,64) -lse2, [64,128) -delta
   __shared__ float red[8];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -275,6 +343,65 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   const int key = kw0 + ln;
   const int key_c = min(key, p.Sk - 1);
   const int64_t kidx = ((int64_t)b * p.Hkv + g) * p.Sk + key_c;
+
+  const int n_qt = (p.Sq + kBK - 1) / kBK;
+  int qt_start = 0;
+  if (p.causal) qt_start = min(max(0, k0 - p.q_start) / kBK, n_qt);
+  const int n_vis = n_qt - qt_start;  // visible query tiles per head
+  const int n_it = n_vis * rep;       // streamed tiles in total
+
+  // ---- staging of one (head, query tile): Qhat and dO tiles plus the two row statistics.
+  // Global addresses are a wave-uniform base (head, tile) plus a per-thread constant offset.
+  constexpr int kStageBytes = 2 * T::kElems * 2;  // one stage = two tiles
+  const int chunk = tid % T::kTPR, srow = tid / T::kTPR;
+  const uint32_t g_off = (uint32_t)(srow * D + chunk * 8) * 2;                  // within a contiguous [64, D] tile
+  const uint32_t l_off = (uint32_t)(srow * T::kRS + chunk * 8) * 2;            // within an LDS tile
+  const bool do_contig = a.do_eff != nullptr;
+  CopyRegs<D> sr;
+  float stat = 0.f;
+  auto tile_load = [&](int it) {
+    const int hq = it / n_vis;
+    const int i0 = (qt_start + it - hq * n_vis) * kBK;
+    const int h = g * rep + hq;
+    const int64_t base = ((int64_t)b * p.H + h) * p.Sq;
+    const char* qsrc = reinterpret_cast<const char*>(a.qhat + (base + i0) * D);
+    const char* dsrc = do_contig ? reinterpret_cast<const char*>(reinterpret_cast<const uint16_t*>(a.do_eff) + (base + i0) * D)
+                                 : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, i0));
+    const uint32_t dstep = do_contig ? (uint32_t)D * 2 : (uint32_t)p.d_o.stride_s * 2;  // bytes between dO rows
+    const uint32_t d_off = (uint32_t)srow * dstep + chunk * 16;
+    if (i0 + kBK <= p.Sq) {
+#pragma unroll
+      for (int ps = 0; ps < T::kPasses; ++ps) {
+        sr.a[ps] = *reinterpret_cast<const u32x4*>(qsrc + g_off + ps * T::kRowsPerPass * D * 2);
+        sr.b[ps] = *reinterpret_cast<const u32x4*>(dsrc + d_off + ps * T::kRowsPerPass * dstep);
+      }
+    } else {  // last tile of a head: rows past Sq are zero-filled
+#pragma unroll
+      for (int ps = 0; ps < T::kPasses; ++ps) {
+        const bool ok = i0 + srow + ps * T::kRowsPerPass < p.Sq;
+        sr.a[ps] = ok ? *reinterpret_cast<const u32x4*>(qsrc + g_off + ps * T::kRowsPerPass * D * 2) : u32x4{0, 0, 0, 0};
+        sr.b[ps] = ok ? *reinterpret_cast<const u32x4*>(dsrc + d_off + ps * T::kRowsPerPass * dstep) : u32x4{0, 0, 0, 0};
+      }
+    }
+    if (tid < 128) {
+      const int i = i0 + (tid & 63);
+      const int64_t ridx = base + min(i, p.Sq - 1);
+      if (tid < 64) stat = i < p.Sq ? -p.lse[ridx] * kLog2e : -INFINITY;  // -inf => P = 0 for padding rows
+      else stat = i < p.Sq ? -a.delta[ridx] : 0.f;
+    }
+  };
+  char* const lds_c = reinterpret_cast<char*>(lds);
+  auto tile_store = [&](int stage) {  // stage is wave-uniform
+    char* qt = lds_c + stage * kStageBytes + l_off;
+#pragma unroll
+    for (int ps = 0; ps < T::kPasses; ++ps) {
+      *reinterpret_cast<u32x4*>(qt + ps * T::kRowsPerPass * T::kRS * 2) = sr.a[ps];
+      *reinterpret_cast<u32x4*>(qt + T::kElems * 2 + ps * T::kRowsPerPass * T::kRS * 2) = sr.b[ps];
+    }
+    if (tid < 128) ldl[stage * 128 + tid] = stat;
+  };
+  if (n_it > 0) { tile_load(0); tile_store(0); }
+  if (n_it > 1) { tile_load(1); tile_store(1); }
 
   // stationary B operands: Khat and V' rows of this lane's key
   bf16x8 kreg[KS], vreg[KS];
@@ -291,96 +418,93 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) { dvacc[mb] = splat16(0.f); dkacc[mb] = splat16(0.f); }
 
-  const int n_qt = (p.Sq + kBK - 1) / kBK;
-  int qt_start = 0;
-  if (p.causal) qt_start = min(max(0, k0 - p.q_start) / kBK, n_qt);
-  const int n_vis = n_qt - qt_start;
-  const int n_it = n_vis * rep;
+  // per-lane LDS bases of stage 0; the running pointers below add the (wave-uniform) stage offset once per
+  // tile, everything else in a fragment address is an immediate
+  const char* const rm_base = lds_c + lane_off_rm<D>(lane);
+  const char* const tr_base = lds_c + lane_off_tr<D>(lane);
+  const float* const st_base = ldl + 4 * hh;
 
-  // staging of one (head, query tile): Qhat and dO tiles plus the two row statistics
-  CopyRegs<D> sr;
-  float stat = 0.f;
-  auto stage_load_q = [&](int hq, int i0) {
-    const int h = g * rep + hq;
-    const int64_t base = ((int64_t)b * p.H + h) * p.Sq;
-    const uint16_t* dbase = a.do_eff ? reinterpret_cast<const uint16_t*>(a.do_eff) + base * D : row_ptr<uint16_t>(p.d_o, b, h, 0);
-    copy_load<D>(a.qhat + base * D, D, dbase, a.do_eff ? (int64_t)D : p.d_o.stride_s, i0, p.Sq, sr);
-    if (tid < 128) {
-      const int i = i0 + (tid & 63);
-      const int64_t ridx = base + min(i, p.Sq - 1);
-      if (tid < 64) stat = i < p.Sq ? -p.lse[ridx] * kLog2e : -INFINITY;  // -inf => P = 0 for padding rows
-      else stat = i < p.Sq ? -a.delta[ridx] : 0.f;
+  bf16x8 qf[KS], df[KS];
+  auto request_rowmajor = [&](const char* rm, int qb) {  // qb is a compile-time constant at every call site
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks] = frag_rm_at<D>(rm, qb, ks);
+      df[ks] = frag_rm_at<D>(rm + T::kElems * 2, qb, ks);
     }
   };
-  auto stage_store_q = [&](int stage) {
-    uint16_t* qt = lds + stage * 2 * T::kElems;
-    copy_store<D>(sr, qt, qt + T::kElems);
-    if (tid < 128) ldl[stage * 128 + tid] = stat;
+  // one 32-query block (qb = 0/1, compile-time) of the tile whose stage the three pointers address;
+  // ib = first query of the block; next_rm = where the following block's row-major fragments live (or null)
+  auto step = [&](const char* rm, const char* tr, const float* st, int qb, int ib, const char* next_rm, int next_qb) {
+    // accumulators of S and dP start from -lse2 / -delta of the 16 query rows their registers map to
+    f32x16 s, dpv;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float4 l4 = *reinterpret_cast<const float4*>(st + 32 * qb + 8 * c);
+      const float4 d4 = *reinterpret_cast<const float4*>(st + 64 + 32 * qb + 8 * c);
+      s[4 * c] = l4.x; s[4 * c + 1] = l4.y; s[4 * c + 2] = l4.z; s[4 * c + 3] = l4.w;
+      dpv[4 * c] = d4.x; dpv[4 * c + 1] = d4.y; dpv[4 * c + 2] = d4.z; dpv[4 * c + 3] = d4.w;
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      s = mfma32(qf[ks], kreg[ks], s);
+      dpv = mfma32(df[ks], vreg[ks], dpv);
+    }
+    bf16x8 dT[MB][2], qT[MB][2];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      dT[mb][0] = frag_tr_at<D>(tr + T::kElems * 2, mb, 2 * qb);
+      qT[mb][0] = frag_tr_at<D>(tr, mb, 2 * qb);
+      dT[mb][1] = frag_tr_at<D>(tr + T::kElems * 2, mb, 2 * qb + 1);
+      qT[mb][1] = frag_tr_at<D>(tr, mb, 2 * qb + 1);
+    }
+    if (p.causal && kw0 + 31 > ib + p.q_start) {  // block touches (or lies above) the diagonal
+      // register r holds query ib + 4hh + c_r with c_r = 8(r/4) + r%4 a compile-time constant:
+      // masked iff key > query + q_start  <=>  key - q_start - ib - 4hh > c_r
+      const int t = key - p.q_start - ib - 4 * hh;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (t > 8 * (r >> 2) + (r & 3)) s[r] = -INFINITY;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      s[r] = fast_exp2(s[r]);
+      dpv[r] *= s[r];
+    }
+    const bf16x8 p0 = pack_c_half(s, 0), p1 = pack_c_half(s, 1);
+    const bf16x8 ds0 = pack_c_half(dpv, 0), ds1 = pack_c_half(dpv, 1);
+    if (next_rm) request_rowmajor(next_rm, next_qb);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      dvacc[mb] = mfma32(dT[mb][0], p0, dvacc[mb]);
+      dkacc[mb] = mfma32(qT[mb][0], ds0, dkacc[mb]);
+      dvacc[mb] = mfma32(dT[mb][1], p1, dvacc[mb]);
+      dkacc[mb] = mfma32(qT[mb][1], ds1, dkacc[mb]);
+    }
   };
 
-  if (n_it > 0) {
-    stage_load_q(0, qt_start * kBK);
-    stage_store_q(0);
-  }
+  // The loads left in flight across the loop must be the YOUNGEST vector-memory operations: every wait
+  // for an older load (the stationary operands above) would otherwise also drain them in each iteration.
+  drain_vector_loads();
+  if (n_it > 2) tile_load(2);
   __syncthreads();
-
+  if (n_it > 0) request_rowmajor(rm_base, 0);
+  int stage = 0;
   for (int it = 0; it < n_it; ++it) {
+    const int nstage = stage == kStages - 1 ? 0 : stage + 1;
     const int hq = it / n_vis;
     const int i0 = (qt_start + it - hq * n_vis) * kBK;
-    const uint16_t* qt = lds + (it & 1) * 2 * T::kElems;
-    const uint16_t* dt = qt + T::kElems;
-    const float* lt = ldl + (it & 1) * 128;
-    const bool more = it + 1 < n_it;
-    if (more) {
-      const int hq2 = (it + 1) / n_vis;
-      stage_load_q(hq2, (qt_start + (it + 1) - hq2 * n_vis) * kBK);
+    const char* rm = rm_base + stage * kStageBytes;
+    const char* tr = tr_base + stage * kStageBytes;
+    const float* st = st_base + stage * 128;
+    const char* rm_next = it + 1 < n_it ? rm_base + nstage * kStageBytes : nullptr;
+    step(rm, tr, st, 0, i0, rm, 1);
+    step(rm, tr, st, 1, i0 + 32, rm_next, 0);
+    if (it + 2 < n_it) {
+      tile_store(nstage == kStages - 1 ? 0 : nstage + 1);
+      if (it + 3 < n_it) tile_load(it + 3);
     }
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      const int ib = i0 + 32 * qb;  // first query of this 32-row block
-      // wave-uniform: is any key of this wave visible to any query of the block?
-      const bool active = ib < p.Sq && (!p.causal || kw0 <= ib + 31 + p.q_start);
-      if (active) {
-        // C operands: -lse2 / -delta of the 16 query rows this lane's registers map to
-        f32x16 s, dpv;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const float4 l4 = *reinterpret_cast<const float4*>(lt + 32 * qb + 8 * c + 4 * hh);
-          const float4 d4 = *reinterpret_cast<const float4*>(lt + 64 + 32 * qb + 8 * c + 4 * hh);
-          s[4 * c] = l4.x; s[4 * c + 1] = l4.y; s[4 * c + 2] = l4.z; s[4 * c + 3] = l4.w;
-          dpv[4 * c] = d4.x; dpv[4 * c + 1] = d4.y; dpv[4 * c + 2] = d4.z; dpv[4 * c + 3] = d4.w;
-        }
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          s = mfma32(frag_rowmajor<D>(qt, qb, ks, lane), kreg[ks], s);
-          dpv = mfma32(frag_rowmajor<D>(dt, qb, ks, lane), vreg[ks], dpv);
-        }
-        const bool need_mask = p.causal && kw0 + 31 > ib + p.q_start;
-        if (need_mask) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int qi = ib + 8 * (r >> 2) + 4 * hh + (r & 3);
-            if (key > qi + p.q_start) s[r] = -INFINITY;
-          }
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          s[r] = fast_exp2(s[r]);
-          dpv[r] *= s[r];
-        }
-        const bf16x8 p0 = pack_c_half(s, 0), p1 = pack_c_half(s, 1);
-        const bf16x8 ds0 = pack_c_half(dpv, 0), ds1 = pack_c_half(dpv, 1);
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-          dvacc[mb] = mfma32(frag_transposed<D>(dt, mb, 2 * qb, lane), p0, dvacc[mb]);
-          dkacc[mb] = mfma32(frag_transposed<D>(qt, mb, 2 * qb, lane), ds0, dkacc[mb]);
-          dvacc[mb] = mfma32(frag_transposed<D>(dt, mb, 2 * qb + 1, lane), p1, dvacc[mb]);
-          dkacc[mb] = mfma32(frag_transposed<D>(qt, mb, 2 * qb + 1, lane), ds1, dkacc[mb]);
-        }
-      }
-    }
-    if (more) stage_store_q((it + 1) & 1);
     __syncthreads();
+    stage = nstage;
   }
 
   // ---- epilogue: lane = key row, registers = head-dim entries

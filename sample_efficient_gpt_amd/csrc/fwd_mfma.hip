@@ -143,11 +143,11 @@ __global__ __launch_bounds__(kThreadsM, 2) void fwd_bf16_kernel(KArgs a) {
 #pragma unroll
           for (int nb = 0; nb < NQB; ++nb) {
             const int qlim = p.causal ? min(qw0 + 32 * nb + ln + p.q_start, p.Sk - 1) : p.Sk - 1;
+            // register r holds key jb + 4hh + c_r, c_r = 8(r/4) + r%4: masked iff c_r > qlim - jb - 4hh
+            const int t = qlim - jb - 4 * hh;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int key = jb + 8 * (r >> 2) + 4 * hh + (r & 3);
-              if (key > qlim) s[nb][r] = -INFINITY;
-            }
+            for (int r = 0; r < 16; ++r)
+              if (8 * (r >> 2) + (r & 3) > t) s[nb][r] = -INFINITY;
           }
         }
         if (!bounded) {

@@ -10,6 +10,8 @@
 // other operand is fetched in exactly that row order ("CPERM order") with two transposing LDS reads.
 #pragma once
 
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace segpt {
@@ -51,6 +53,15 @@ __device__ __forceinline__ float half_sum(float x) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// Wait for every outstanding vector-memory load of this wave and keep the compiler from moving memory
+// operations across this point.  Used once before a pipelined loop: loads that stay in flight ACROSS loop
+// iterations must be the youngest ones, or every in-loop wait for an older load drains them as well.
+__device__ __forceinline__ void drain_vector_loads() {
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt/lgkmcnt untouched
+  __builtin_amdgcn_sched_barrier(0);
+}
 
 // x + (x of another lane) through a DPP lane pattern (no LDS traffic, fuses into v_add_f32_dpp)
 template <int CTRL>
@@ -129,6 +140,35 @@ __device__ __forceinline__ bf16x8 frag_transposed(const uint16_t* tile, int cb, 
   s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   return __builtin_bit_cast(bf16x8, v);
 }
+
+// ---- the same two fragment readers with every term but one per-lane base folded into the instruction's
+// immediate offset: `base` = LDS byte address of the tile + lane_off_rm / lane_off_tr, block indices constant.
+template <int D>
+__device__ __forceinline__ int lane_off_rm(int lane) {
+  return ((lane & 31) * Tile<D>::kRS + 8 * (lane >> 5)) * 2;
+}
+template <int D>
+__device__ __forceinline__ int lane_off_tr(int lane) {
+  const int r = lane & 15;
+  return ((4 * (lane >> 5) + (r >> 2)) * Tile<D>::kRS + 16 * ((lane >> 4) & 1) + 4 * (r & 3)) * 2;
+}
+template <int D>
+__device__ __forceinline__ bf16x8 frag_rm_at(const char* base, int rb, int ks) {
+  return as_bf16x8(*reinterpret_cast<const u32x4*>(base + (32 * rb * Tile<D>::kRS + 16 * ks) * 2));
+}
+template <int D>
+__device__ __forceinline__ bf16x8 frag_tr_at(const char* base, int cb, int s) {
+  const char* p = base + (16 * s * Tile<D>::kRS + 32 * cb) * 2;
+  typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 8 * Tile<D>::kRS * 2));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+template <int N>
+using IC = std::integral_constant<int, N>;
 
 // pack registers 8s..8s+7 of a C tile into a bf16 operand (CPERM order)
 __device__ __forceinline__ bf16x8 pack_c_half(const f32x16& c, int s) {

@@ -17,57 +17,66 @@ __global__ __launch_bounds__(256) void bwd_pre_kernel(KArgs a) {
   const segpt_attn_params& p = a.p;
   constexpr int V = Elem<T>::kVec;
   constexpr int TPR = D / V;          // threads per row
-  constexpr int RPB = 256 / TPR;      // rows per block
+  constexpr int RPB = 256 / TPR;      // rows per pass of a block
   const int tid = threadIdx.x;
   const int part = tid % TPR;
-  const int64_t rid = (int64_t)blockIdx.x * RPB + tid / TPR;  // flat (b, h, s)
   const int64_t nrows = (int64_t)p.B * p.H * p.Sq;
-  const bool live = rid < nrows;
-  const int64_t r = live ? rid : nrows - 1;
-  const int s = (int)(r % p.Sq);
-  const int h = (int)((r / p.Sq) % p.H);
-  const int b = (int)(r / ((int64_t)p.Sq * p.H));
-  float y[V], dy[V];
-  Elem<T>::load(row_ptr<T>(p.o, b, h, s) + part * V, y);
-  Elem<T>::load(row_ptr<T>(p.d_o, b, h, s) + part * V, dy);
-  float acc = 0.f;
-#pragma unroll
-  for (int e = 0; e < V; ++e) acc += y[e] * dy[e];
-#pragma unroll
-  for (int o = 1; o < TPR; o <<= 1) acc += __shfl_xor(acc, o, 64);
-  if (a.qhat) {  // bf16 path: the normalised, scaled query row the two MFMA kernels consume
-    float q[V];
-    Elem<T>::load(row_ptr<T>(p.q, b, h, s) + part * V, q);
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < V; ++e) ss += q[e] * q[e];
-#pragma unroll
-    for (int o = 1; o < TPR; o <<= 1) ss += __shfl_xor(ss, o, 64);
-    const float f = (1.0f / sqrtf(ss * (1.0f / D) + p.eps)) * p.sm_scale * kLog2e;
+  // the slice of the scale product this thread needs when it forms Qhat (bf16 path)
+  float gs[V];
+  if (a.qhat) {
 #pragma unroll
     for (int e = 0; e < V; ++e) {
       const int d = part * V + e;
       float g = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
       if (p.gk_numel == 1) g *= p.g_k[0];
       else if (p.gk_numel > 1) g *= p.g_k[d];
-      q[e] *= f * g;
+      gs[e] = g * p.sm_scale * kLog2e;
     }
-    if (live) Elem<T>::store(reinterpret_cast<T*>(a.qhat) + r * D + part * V, q);
   }
-  if (!live) return;
-  if (part == 0) a.delta[r] = acc;
-  if (p.gate.ptr) {
-    const int64_t gi = (int64_t)b * p.gate.stride_b + (int64_t)s * p.gate.stride_s + (int64_t)h * p.gate.stride_h;
-    const float z = Elem<T>::load1(reinterpret_cast<const T*>(p.gate.ptr) + gi);
-    const float sg = sigmoidf_acc(z);
-    if (part == 0) {
-      const int64_t di = (int64_t)b * p.dgate.stride_b + (int64_t)s * p.dgate.stride_s + (int64_t)h * p.dgate.stride_h;
-      Elem<T>::store1(reinterpret_cast<T*>(p.dgate.ptr) + di, (1.0f - sg) * acc);
-    }
-    const float f = p.gate_scale * sg;
+  for (int64_t row0 = (int64_t)blockIdx.x * RPB; row0 < nrows; row0 += (int64_t)gridDim.x * RPB) {
+    const int64_t rid = row0 + tid / TPR;  // flat (b, h, s)
+    const bool live = rid < nrows;
+    const int64_t r = live ? rid : nrows - 1;
+    const int s = (int)(r % p.Sq);
+    const int h = (int)((r / p.Sq) % p.H);
+    const int b = (int)(r / ((int64_t)p.Sq * p.H));
+    float y[V], dy[V], q[V];
+    Elem<T>::load(row_ptr<T>(p.o, b, h, s) + part * V, y);
+    Elem<T>::load(row_ptr<T>(p.d_o, b, h, s) + part * V, dy);
+    if (a.qhat) Elem<T>::load(row_ptr<T>(p.q, b, h, s) + part * V, q);
+    float acc = 0.f, ss = 0.f;
 #pragma unroll
-    for (int e = 0; e < V; ++e) dy[e] *= f;
-    Elem<T>::store(reinterpret_cast<T*>(a.do_eff) + r * D + part * V, dy);
+    for (int e = 0; e < V; ++e) acc += y[e] * dy[e];
+    if (a.qhat) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) ss += q[e] * q[e];
+    }
+#pragma unroll
+    for (int o = 1; o < TPR; o <<= 1) {
+      acc += __shfl_xor(acc, o, 64);
+      ss += __shfl_xor(ss, o, 64);
+    }
+    if (!live) continue;
+    if (a.qhat) {  // bf16 path: the normalised, scaled query row the two MFMA kernels consume
+      const float f = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
+#pragma unroll
+      for (int e = 0; e < V; ++e) q[e] *= f * gs[e];
+      Elem<T>::store(reinterpret_cast<T*>(a.qhat) + r * D + part * V, q);
+    }
+    if (part == 0) a.delta[r] = acc;
+    if (p.gate.ptr) {
+      const int64_t gi = (int64_t)b * p.gate.stride_b + (int64_t)s * p.gate.stride_s + (int64_t)h * p.gate.stride_h;
+      const float z = Elem<T>::load1(reinterpret_cast<const T*>(p.gate.ptr) + gi);
+      const float sg = sigmoidf_acc(z);
+      if (part == 0) {
+        const int64_t di = (int64_t)b * p.dgate.stride_b + (int64_t)s * p.dgate.stride_s + (int64_t)h * p.dgate.stride_h;
+        Elem<T>::store1(reinterpret_cast<T*>(p.dgate.ptr) + di, (1.0f - sg) * acc);
+      }
+      const float f = p.gate_scale * sg;
+#pragma unroll
+      for (int e = 0; e < V; ++e) dy[e] *= f;
+      Elem<T>::store(reinterpret_cast<T*>(a.do_eff) + r * D + part * V, dy);
+    }
   }
 }
 
@@ -118,19 +127,20 @@ __global__ __launch_bounds__(kReduceThreads) void bwd_reduce_kernel(KArgs a) {
   const int D = p.D;
   const int lanes = kReduceThreads / D;  // threads cooperating on one d
   const int d = tid % D, sl = tid / D;
-  // fixed summation order (deterministic); four independent chains hide the load latency
-  float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+  // fixed summation order (deterministic); eight independent chains hide the load latency
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const float* src = a.dg_part + d;
   const int n = a.n_dq_blocks;
   int blk = sl;
-  for (; blk + 3 * lanes < n; blk += 4 * lanes) {
-    acc0 += src[(int64_t)blk * D];
-    acc1 += src[(int64_t)(blk + lanes) * D];
-    acc2 += src[(int64_t)(blk + 2 * lanes) * D];
-    acc3 += src[(int64_t)(blk + 3 * lanes) * D];
+  for (; blk + 7 * lanes < n; blk += 8 * lanes) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(blk + u * lanes) * D];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc[u] += v[u];
   }
-  for (; blk < n; blk += lanes) acc0 += src[(int64_t)blk * D];
-  red[tid] = (acc0 + acc1) + (acc2 + acc3);
+  for (; blk < n; blk += lanes) acc[0] += src[(int64_t)blk * D];
+  red[tid] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
   __syncthreads();
   if (tid < D) {
     float t = 0.f;
@@ -191,7 +201,8 @@ int launch_pre_t(const KArgs& a, hipStream_t st) {
   const int64_t nrows = (int64_t)p.B * p.H * p.Sq;
   constexpr int V = Elem<T>::kVec;
   const int rpb = 256 / (p.D / V);
-  dim3 grid((unsigned)((nrows + rpb - 1) / rpb)), block(256);
+  const int64_t groups = (nrows + rpb - 1) / rpb;
+  dim3 grid((unsigned)(groups < 8192 ? groups : 8192)), block(256);  // grid-stride: <= 32 blocks per CU
   switch (p.D) {
     case 32:
       if constexpr (sizeof(T) == 4) { hipLaunchKernelGGL((bwd_pre_kernel<T, 32>), grid, block, 0, st, a); break; }
@@ -207,8 +218,7 @@ int launch_pre_t(const KArgs& a, hipStream_t st) {
 
 int launch_bwd_pre(const KArgs& a, hipStream_t st) {
   if (a.p.dtype == SEGPT_DTYPE_FP32) return launch_pre_t<float>(a, st);
-  int rc = launch_pre_t<uint16_t>(a, st);
-  if (rc) return rc;
+  // bf16: the per-query-row quantities (delta, Qhat, gate terms) come from the dQ kernel's prologue
   const segpt_attn_params& p = a.p;
   const int64_t nrows = (int64_t)p.B * p.Hkv * p.Sk;
   const int rpb = 256 / (p.D / 8);
