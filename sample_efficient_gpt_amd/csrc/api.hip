@@ -23,7 +23,7 @@ size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 size_t elem_bytes(const segpt_attn_params& p) { return p.dtype == SEGPT_DTYPE_FP32 ? 4 : 2; }
 
 struct WsLayout {
-  size_t delta, do_eff, qhat, khat, vmix, dg_part, dcoef_part, total;
+  size_t delta, nlse2, do_eff, qhat, khat, vmix, dg_part, dcoef_part, total;
 };
 
 WsLayout bwd_layout(const segpt_attn_params& p) {
@@ -32,6 +32,8 @@ WsLayout bwd_layout(const segpt_attn_params& p) {
   const size_t rows = (size_t)p.B * p.H * p.Sq;
   w.delta = off;
   off += align_up(rows * sizeof(float));
+  w.nlse2 = off;
+  if (p.dtype == SEGPT_DTYPE_BF16) off += align_up(rows * sizeof(float));
   w.do_eff = off;
   if (p.gate.ptr) off += align_up(rows * p.D * elem_bytes(p));
   w.qhat = w.khat = w.vmix = off;
@@ -169,6 +171,7 @@ static int bwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi
   a.dg_part = reinterpret_cast<float*>(ws + w.dg_part);
   a.dcoef_part = reinterpret_cast<float*>(ws + w.dcoef_part);
   if (p->dtype == SEGPT_DTYPE_BF16) {
+    a.nlse2 = reinterpret_cast<float*>(ws + w.nlse2);
     a.qhat = reinterpret_cast<uint16_t*>(ws + w.qhat);
     a.khat = reinterpret_cast<uint16_t*>(ws + w.khat);
     a.vmix = p->v_first.ptr ? reinterpret_cast<uint16_t*>(ws + w.vmix) : nullptr;

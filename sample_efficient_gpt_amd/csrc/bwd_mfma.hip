@@ -61,43 +61,6 @@ __device__ __forceinline__ void load_ct_block(const uint16_t* rowp, int mb, int 
   }
 }
 
-// ---- staging of two row-major bf16 tiles (64 rows x D) that need no arithmetic: global -> regs -> LDS
-template <int D>
-struct CopyRegs {
-  u32x4 a[Tile<D>::kPasses], b[Tile<D>::kPasses];
-};
-// rows r0.. of two tensors with the same (contiguous, stride D) layout starting at base pointers pa, pb
-template <int D>
-__device__ __forceinline__ void copy_load(const uint16_t* pa, int64_t stride_a, const uint16_t* pb, int64_t stride_b,
-                                          int row0, int nrows, CopyRegs<D>& r) {
-  using T = Tile<D>;
-  const int tid = threadIdx.x;
-  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
-#pragma unroll
-  for (int ps = 0; ps < T::kPasses; ++ps) {
-    const int i = row0 + r0 + ps * T::kRowsPerPass;
-    if (i < nrows) {
-      r.a[ps] = *reinterpret_cast<const u32x4*>(pa + (int64_t)i * stride_a + chunk * 8);
-      r.b[ps] = *reinterpret_cast<const u32x4*>(pb + (int64_t)i * stride_b + chunk * 8);
-    } else {
-      r.a[ps] = u32x4{0, 0, 0, 0};
-      r.b[ps] = u32x4{0, 0, 0, 0};
-    }
-  }
-}
-template <int D>
-__device__ __forceinline__ void copy_store(const CopyRegs<D>& r, uint16_t* ta, uint16_t* tb) {
-  using T = Tile<D>;
-  const int tid = threadIdx.x;
-  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
-#pragma unroll
-  for (int ps = 0; ps < T::kPasses; ++ps) {
-    const int row = r0 + ps * T::kRowsPerPass;
-    *reinterpret_cast<u32x4*>(ta + row * T::kRS + chunk * 8) = r.a[ps];
-    *reinterpret_cast<u32x4*>(tb + row * T::kRS + chunk * 8) = r.b[ps];
-  }
-}
-
 __device__ __forceinline__ f32x16 splat16(float x) {
   f32x16 v;
 #pragma unroll
@@ -105,11 +68,27 @@ __device__ __forceinline__ f32x16 splat16(float x) {
   return v;
 }
 
-constexpr int kStages = 3;  // LDS ring of streamed tiles: tile t lives in stage t % 3
+constexpr int kStages = 4;  // LDS ring of streamed stages (two tiles each): tile t lives in stage t % 4
+
+// Issue the direct global->LDS loads of two [64, D] bf16 tiles (rows row0..row0+63 of two row-major
+// tensors; rows past nrows re-read the last valid row, callers mask them) into one stage.
+//   src_a/src_b: wave-uniform pointers to row `row0` of each tensor; step_*: bytes between rows
+//   dst: LDS byte address of the stage + wave*1024 (wave-uniform); lane_row / lane_col: from swz_src()
+template <int D>
+__device__ __forceinline__ void issue_tile_pair(const char* src_a, uint32_t step_a, const char* src_b, uint32_t step_b,
+                                                int rows_left, uint32_t dst, int lane_row, int lane_col) {
+  using Z = Swz<D>;
+#pragma unroll
+  for (int ps = 0; ps < Z::kPasses; ++ps) {
+    const int row = min(lane_row + ps * 4 * Z::kRowsPerInst, rows_left - 1);
+    gload_lds16(src_a + (uint32_t)row * step_a + lane_col, dst + ps * 4096);
+    gload_lds16(src_b + (uint32_t)row * step_b + lane_col, dst + Z::kTileBytes + ps * 4096);
+  }
+}
 
 // ============================================================================================ dQ
-// Also the producer of the per-query-row quantities the dK/dV kernel streams afterwards: Qhat, delta
-// and (with a gate) the gate-scaled dO and dgate.
+// Also the producer of the per-query-row quantities the dK/dV kernel streams afterwards: Qhat, -delta,
+// -lse*log2e and (with a gate) the gate-scaled dO and dgate.
 //
 // Software pipeline over 32-key blocks n (two per staged tile), one barrier per tile:
 //   B(n)  S^T, dP^T MFMAs from the row-major fragments requested one block earlier
@@ -117,16 +96,18 @@ constexpr int kStages = 3;  // LDS ring of streamed tiles: tile t lives in stage
 //   D(n)  dS^T = exp2(S^T) * dP^T, pack to bf16
 //   A(n+1) request the row-major fragments of block n+1 (possibly the next tile, already in LDS)
 //   E(n)  T^T += Khat^T dS^T MFMAs
-// Tiles are stored two tiles ahead of their use so that A(n+1) never waits for a barrier.
+// Tiles travel global->LDS directly (no registers), three tiles ahead of their use.
 template <int D>
 __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel(KArgs a) {
-  using T = Tile<D>;
+  using Z = Swz<D>;
   constexpr int BQ = kBwdRows;
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
+  constexpr int kStageBytes = 2 * Z::kTileBytes;
+  constexpr int kLoadsPerTile = 2 * Z::kPasses;  // per wave
   const segpt_attn_params& p = a.p;
-  __shared__ __attribute__((aligned(16))) uint16_t lds[kStages * 2 * T::kElems];
-  static_assert(kStages * 2 * T::kElems * 2 >= 128 * (D + 1) * 4, "LDS reuse for the dg partial");
+  __shared__ __attribute__((aligned(1024))) char lds[kStages * kStageBytes];
+  static_assert(kStages * kStageBytes >= 128 * (D + 1) * 4, "LDS reuse for the dg partial");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, hh = lane >> 5;
@@ -144,18 +125,18 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   int kend = p.Sk;
   if (p.causal) kend = min(p.Sk, q0 + BQ + p.q_start);
   const int n_kt = (kend + kBK - 1) / kBK;
-  const uint16_t* kbase = a.khat + ((int64_t)b * p.Hkv + g) * p.Sk * D;
-  const uint16_t* vbase = a.vmix ? a.vmix + ((int64_t)b * p.Hkv + g) * p.Sk * D : row_ptr<uint16_t>(p.v, b, g, 0);
-  const int64_t vstride = a.vmix ? D : p.v.stride_s;
+  const char* kbase = reinterpret_cast<const char*>(a.khat + ((int64_t)b * p.Hkv + g) * p.Sk * D);
+  const char* vbase = a.vmix ? reinterpret_cast<const char*>(a.vmix + ((int64_t)b * p.Hkv + g) * p.Sk * D)
+                             : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.v, b, g, 0));
+  const uint32_t kstep = D * 2, vstep = a.vmix ? (uint32_t)D * 2 : (uint32_t)p.v.stride_s * 2;
 
-  // ---- first two tiles on their way to LDS while the query-row prologue runs
-  CopyRegs<D> sr;
-  copy_load<D>(kbase, D, vbase, vstride, 0, p.Sk, sr);
-  copy_store<D>(sr, lds, lds + T::kElems);
-  if (n_kt > 1) {
-    copy_load<D>(kbase, D, vbase, vstride, kBK, p.Sk, sr);
-    copy_store<D>(sr, lds + 2 * T::kElems, lds + 3 * T::kElems);
-  }
+  const uint32_t lds0 = lds_addr_of(lds);
+  const int2 src = swz_src<D>(lane, wave);
+  const uint32_t wave_dst = lds0 + __builtin_amdgcn_readfirstlane(wave) * 1024;
+  auto issue_tile = [&](int jt) {  // tile jt -> stage jt % kStages
+    issue_tile_pair<D>(kbase + (int64_t)jt * kBK * kstep, kstep, vbase + (int64_t)jt * kBK * vstep, vstep,
+                       p.Sk - jt * kBK, wave_dst + (jt % kStages) * kStageBytes, src.x, src.y);
+  };
 
   // ---- query-row prologue: alpha, Qhat, delta, gate; B operands stay in registers
   bf16x8 qreg[KS], doreg[KS];
@@ -205,10 +186,12 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
         doreg[ks] = as_bf16x8(dyraw[ks]);
       }
     }
-    if (live && hh == 0) a.delta[ridx] = delta;
   }
-  // row statistics as MFMA C operands (every register of a lane belongs to the lane's query)
-  const f32x16 c_lse = splat16(-p.lse[ridx] * kLog2e);
+  // row statistics as MFMA C operands (every register of a lane belongs to the lane's query); the dK/dV
+  // kernel reads the same two numbers per row from the workspace
+  const float nlse2 = -p.lse[ridx] * kLog2e;
+  if (live && hh == 0) { a.delta[ridx] = -delta; a.nlse2[ridx] = nlse2; }
+  const f32x16 c_lse = splat16(nlse2);
   const f32x16 c_del = splat16(-delta);
 
   f32x16 acc[MB];
@@ -216,23 +199,23 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   for (int mb = 0; mb < MB; ++mb) acc[mb] = splat16(0.f);
 
   // blocks this wave has to visit (causal: up to the block holding its last query's diagonal)
-  int n_act = (min(kend, p.Sk) + 31) / 32;
+  int n_act = (kend + 31) / 32;
   if (p.causal) n_act = min(n_act, (qw0 + 31 + p.q_start) / 32 + 1);
   const int qlim = p.causal ? min(row + p.q_start, p.Sk - 1) : p.Sk - 1;  // last visible key of this lane's query
 
+  const uint32_t rm_lane = lds0 + swz_off_rm<D>(lane);
+  const uint32_t tr_lane = lds0 + swz_off_tr<D>(lane);
   bf16x8 kf[KS], vf[KS];
-  auto request_rowmajor = [&](int blk) {
-    const uint16_t* kt = lds + ((blk >> 1) % kStages) * 2 * T::kElems;
+  auto request_rowmajor = [&](uint32_t rm, int kb) {  // kb compile-time at every call site
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      kf[ks] = frag_rowmajor<D>(kt, blk & 1, ks, lane);
-      vf[ks] = frag_rowmajor<D>(kt + T::kElems, blk & 1, ks, lane);
+      kf[ks] = swz_frag_rm<D>(rm, kb, ks);
+      vf[ks] = swz_frag_rm<D>(rm + Z::kTileBytes, kb, ks);
     }
   };
-  auto step = [&](int blk) {
-    const uint16_t* kt = lds + ((blk >> 1) % kStages) * 2 * T::kElems;
-    const int kb = blk & 1;
-    const int jb = blk * 32;
+  // one 32-key block: tr = lane address inside the block's stage; `more`: a block follows, its row-major
+  // fragments start at next_rm
+  auto step = [&](uint32_t tr, int kb, int jb, bool more, uint32_t next_rm, int next_kb) {
     f32x16 s = c_lse, dpv = c_del;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -242,8 +225,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     bf16x8 kT[MB][2];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      kT[mb][0] = frag_transposed<D>(kt, mb, 2 * kb, lane);
-      kT[mb][1] = frag_transposed<D>(kt, mb, 2 * kb + 1, lane);
+      kT[mb][0] = swz_frag_tr<D>(tr, mb, 2 * kb);
+      kT[mb][1] = swz_frag_tr<D>(tr, mb, 2 * kb + 1);
     }
     if ((p.causal && jb + 31 > qw0 + p.q_start) || jb + 32 > p.Sk) {  // block touches the diagonal or the end of the keys
       // register r holds key jb + 4hh + c_r, c_r = 8(r/4) + r%4: masked iff c_r > qlim - jb - 4hh
@@ -255,7 +238,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = fast_exp2(s[r]) * dpv[r];
     const bf16x8 ds0 = pack_c_half(s, 0), ds1 = pack_c_half(s, 1);
-    if (blk + 1 < n_act) request_rowmajor(blk + 1);
+    if (more) request_rowmajor(next_rm, next_kb);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       acc[mb] = mfma32(kT[mb][0], ds0, acc[mb]);
@@ -263,21 +246,27 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     }
   };
 
-  // The loads left in flight across the loop must be the YOUNGEST vector-memory operations: every wait
-  // for an older load (the row prologue above) would otherwise also drain them in each iteration.
+  // ---- pipeline start-up.  All earlier vector loads are drained first: the tile loads that stay in flight
+  // across iterations must be the youngest vector-memory operations of the wave (waits are in-order).
   drain_vector_loads();
-  if (n_kt > 2) copy_load<D>(kbase, D, vbase, vstride, 2 * kBK, p.Sk, sr);
+  issue_tile(0);
+  if (n_kt > 1) issue_tile(1);
+  if (n_kt > 2) issue_tile(2);
+  if (n_kt > 2) wait_vmcnt<kLoadsPerTile>(); else wait_vmcnt<0>();  // tiles 0 and 1 have landed
   __syncthreads();
-  if (n_act > 0) request_rowmajor(0);
+  if (n_act > 0) request_rowmajor(rm_lane, 0);
+  int stage = 0;
   for (int jt = 0; jt < n_kt; ++jt) {
-    if (2 * jt < n_act) step(2 * jt);
-    if (2 * jt + 1 < n_act) step(2 * jt + 1);
-    if (jt + 2 < n_kt) {
-      uint16_t* nk = lds + ((jt + 2) % kStages) * 2 * T::kElems;
-      copy_store<D>(sr, nk, nk + T::kElems);
-      if (jt + 3 < n_kt) copy_load<D>(kbase, D, vbase, vstride, (jt + 3) * kBK, p.Sk, sr);
-    }
+    const int nstage = stage == kStages - 1 ? 0 : stage + 1;
+    const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
+    const uint32_t rm_next = rm_lane + nstage * kStageBytes;
+    if (2 * jt < n_act) step(tr, 0, 64 * jt, 2 * jt + 1 < n_act, rm, 1);
+    if (2 * jt + 1 < n_act) step(tr, 1, 64 * jt + 32, 2 * jt + 2 < n_act, rm_next, 0);
+    // stage (jt+3) % 4 == (jt-1) % 4 was last read in the previous iteration: refill it, then make sure
+    // this wave's part of tile jt+2 (needed from the next iteration's prefetch on) has landed
+    if (jt + 3 < n_kt) { issue_tile(jt + 3); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
     __syncthreads();
+    stage = nstage;
   }
 
   // ---- epilogue.  acc = T^T: lane = query, registers = head-dim entries.
@@ -322,13 +311,15 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
 // straight into the accumulators of S and dP.
 template <int D>
 __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kernel(KArgs a) {
-  using T = Tile<D>;
+  using Z = Swz<D>;
   constexpr int BKV = kBwdRows;
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
+  constexpr int kStageBytes = 2 * Z::kTileBytes;
+  constexpr int kLoadsPerTile = 2 * Z::kPasses + 1;  // per wave: the two tiles plus one row-statistics load
   const segpt_attn_params& p = a.p;
-  __shared__ __attribute__((aligned(16))) uint16_t lds[kStages * 2 * T::kElems];
-  __shared__ __attribute__((aligned(16))) float ldl[kStages * 128];  // per stage: [0,64) -lse2, [64,128) -delta
+  __shared__ __attribute__((aligned(1024))) char lds[kStages * kStageBytes];
+  __shared__ __attribute__((aligned(256))) float ldl[kStages * 128];  // per stage: [0,64) -lse2, [64,128) -delta
   __shared__ float red[8];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -350,16 +341,15 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   const int n_vis = n_qt - qt_start;  // visible query tiles per head
   const int n_it = n_vis * rep;       // streamed tiles in total
 
-  // ---- staging of one (head, query tile): Qhat and dO tiles plus the two row statistics.
-  // Global addresses are a wave-uniform base (head, tile) plus a per-thread constant offset.
-  constexpr int kStageBytes = 2 * T::kElems * 2;  // one stage = two tiles
-  const int chunk = tid % T::kTPR, srow = tid / T::kTPR;
-  const uint32_t g_off = (uint32_t)(srow * D + chunk * 8) * 2;                  // within a contiguous [64, D] tile
-  const uint32_t l_off = (uint32_t)(srow * T::kRS + chunk * 8) * 2;            // within an LDS tile
+  // ---- staging of one (head, query tile): Qhat and dO tiles plus the two row statistics, all by direct
+  // global->LDS loads.  Every wave issues the same number of loads (waves 2/3 repeat the statistics load
+  // of waves 0/1) so that one immediate vmcnt fits all.
+  const uint32_t lds0 = lds_addr_of(lds), ldl0 = lds_addr_of(ldl);
+  const int2 src = swz_src<D>(lane, wave);
+  const int uwave = __builtin_amdgcn_readfirstlane(wave);
   const bool do_contig = a.do_eff != nullptr;
-  CopyRegs<D> sr;
-  float stat = 0.f;
-  auto tile_load = [&](int it) {
+  const float* const stat_arr = (uwave & 1) ? a.delta : a.nlse2;
+  auto issue_tile = [&](int it) {  // streamed tile it -> stage it % kStages
     const int hq = it / n_vis;
     const int i0 = (qt_start + it - hq * n_vis) * kBK;
     const int h = g * rep + hq;
@@ -367,41 +357,11 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     const char* qsrc = reinterpret_cast<const char*>(a.qhat + (base + i0) * D);
     const char* dsrc = do_contig ? reinterpret_cast<const char*>(reinterpret_cast<const uint16_t*>(a.do_eff) + (base + i0) * D)
                                  : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, i0));
-    const uint32_t dstep = do_contig ? (uint32_t)D * 2 : (uint32_t)p.d_o.stride_s * 2;  // bytes between dO rows
-    const uint32_t d_off = (uint32_t)srow * dstep + chunk * 16;
-    if (i0 + kBK <= p.Sq) {
-#pragma unroll
-      for (int ps = 0; ps < T::kPasses; ++ps) {
-        sr.a[ps] = *reinterpret_cast<const u32x4*>(qsrc + g_off + ps * T::kRowsPerPass * D * 2);
-        sr.b[ps] = *reinterpret_cast<const u32x4*>(dsrc + d_off + ps * T::kRowsPerPass * dstep);
-      }
-    } else {  // last tile of a head: rows past Sq are zero-filled
-#pragma unroll
-      for (int ps = 0; ps < T::kPasses; ++ps) {
-        const bool ok = i0 + srow + ps * T::kRowsPerPass < p.Sq;
-        sr.a[ps] = ok ? *reinterpret_cast<const u32x4*>(qsrc + g_off + ps * T::kRowsPerPass * D * 2) : u32x4{0, 0, 0, 0};
-        sr.b[ps] = ok ? *reinterpret_cast<const u32x4*>(dsrc + d_off + ps * T::kRowsPerPass * dstep) : u32x4{0, 0, 0, 0};
-      }
-    }
-    if (tid < 128) {
-      const int i = i0 + (tid & 63);
-      const int64_t ridx = base + min(i, p.Sq - 1);
-      if (tid < 64) stat = i < p.Sq ? -p.lse[ridx] * kLog2e : -INFINITY;  // -inf => P = 0 for padding rows
-      else stat = i < p.Sq ? -a.delta[ridx] : 0.f;
-    }
+    const uint32_t dstep = do_contig ? (uint32_t)D * 2 : (uint32_t)p.d_o.stride_s * 2;
+    const int stage = it % kStages;
+    issue_tile_pair<D>(qsrc, D * 2, dsrc, dstep, p.Sq - i0, lds0 + stage * kStageBytes + uwave * 1024, src.x, src.y);
+    gload_lds4(stat_arr + base + min(i0 + lane, p.Sq - 1), ldl0 + (stage * 128 + (uwave & 1) * 64) * 4);
   };
-  char* const lds_c = reinterpret_cast<char*>(lds);
-  auto tile_store = [&](int stage) {  // stage is wave-uniform
-    char* qt = lds_c + stage * kStageBytes + l_off;
-#pragma unroll
-    for (int ps = 0; ps < T::kPasses; ++ps) {
-      *reinterpret_cast<u32x4*>(qt + ps * T::kRowsPerPass * T::kRS * 2) = sr.a[ps];
-      *reinterpret_cast<u32x4*>(qt + T::kElems * 2 + ps * T::kRowsPerPass * T::kRS * 2) = sr.b[ps];
-    }
-    if (tid < 128) ldl[stage * 128 + tid] = stat;
-  };
-  if (n_it > 0) { tile_load(0); tile_store(0); }
-  if (n_it > 1) { tile_load(1); tile_store(1); }
 
   // stationary B operands: Khat and V' rows of this lane's key
   bf16x8 kreg[KS], vreg[KS];
@@ -418,31 +378,29 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) { dvacc[mb] = splat16(0.f); dkacc[mb] = splat16(0.f); }
 
-  // per-lane LDS bases of stage 0; the running pointers below add the (wave-uniform) stage offset once per
-  // tile, everything else in a fragment address is an immediate
-  const char* const rm_base = lds_c + lane_off_rm<D>(lane);
-  const char* const tr_base = lds_c + lane_off_tr<D>(lane);
-  const float* const st_base = ldl + 4 * hh;
+  const uint32_t rm_lane = lds0 + swz_off_rm<D>(lane);
+  const uint32_t tr_lane = lds0 + swz_off_tr<D>(lane);
+  const uint32_t st_lane = ldl0 + 16 * hh;
 
   bf16x8 qf[KS], df[KS];
-  auto request_rowmajor = [&](const char* rm, int qb) {  // qb is a compile-time constant at every call site
+  auto request_rowmajor = [&](uint32_t rm, int qb) {  // qb is a compile-time constant at every call site
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      qf[ks] = frag_rm_at<D>(rm, qb, ks);
-      df[ks] = frag_rm_at<D>(rm + T::kElems * 2, qb, ks);
+      qf[ks] = swz_frag_rm<D>(rm, qb, ks);
+      df[ks] = swz_frag_rm<D>(rm + Z::kTileBytes, qb, ks);
     }
   };
-  // one 32-query block (qb = 0/1, compile-time) of the tile whose stage the three pointers address;
-  // ib = first query of the block; next_rm = where the following block's row-major fragments live (or null)
-  auto step = [&](const char* rm, const char* tr, const float* st, int qb, int ib, const char* next_rm, int next_qb) {
+  // one 32-query block (qb = 0/1, compile-time) of the tile whose stage the pointers address;
+  // ib = first query of the block; `more`: a block follows, its row-major fragments start at next_rm
+  auto step = [&](uint32_t tr, uint32_t st, int qb, int ib, bool more, uint32_t next_rm, int next_qb) {
     // accumulators of S and dP start from -lse2 / -delta of the 16 query rows their registers map to
     f32x16 s, dpv;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      const float4 l4 = *reinterpret_cast<const float4*>(st + 32 * qb + 8 * c);
-      const float4 d4 = *reinterpret_cast<const float4*>(st + 64 + 32 * qb + 8 * c);
-      s[4 * c] = l4.x; s[4 * c + 1] = l4.y; s[4 * c + 2] = l4.z; s[4 * c + 3] = l4.w;
-      dpv[4 * c] = d4.x; dpv[4 * c + 1] = d4.y; dpv[4 * c + 2] = d4.z; dpv[4 * c + 3] = d4.w;
+      const f32x4 l4 = lds_read_f4(st + (32 * qb + 8 * c) * 4);
+      const f32x4 d4 = lds_read_f4(st + (64 + 32 * qb + 8 * c) * 4);
+      s[4 * c] = l4[0]; s[4 * c + 1] = l4[1]; s[4 * c + 2] = l4[2]; s[4 * c + 3] = l4[3];
+      dpv[4 * c] = d4[0]; dpv[4 * c + 1] = d4[1]; dpv[4 * c + 2] = d4[2]; dpv[4 * c + 3] = d4[3];
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -452,18 +410,21 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     bf16x8 dT[MB][2], qT[MB][2];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      dT[mb][0] = frag_tr_at<D>(tr + T::kElems * 2, mb, 2 * qb);
-      qT[mb][0] = frag_tr_at<D>(tr, mb, 2 * qb);
-      dT[mb][1] = frag_tr_at<D>(tr + T::kElems * 2, mb, 2 * qb + 1);
-      qT[mb][1] = frag_tr_at<D>(tr, mb, 2 * qb + 1);
+      dT[mb][0] = swz_frag_tr<D>(tr + Z::kTileBytes, mb, 2 * qb);
+      qT[mb][0] = swz_frag_tr<D>(tr, mb, 2 * qb);
+      dT[mb][1] = swz_frag_tr<D>(tr + Z::kTileBytes, mb, 2 * qb + 1);
+      qT[mb][1] = swz_frag_tr<D>(tr, mb, 2 * qb + 1);
     }
-    if (p.causal && kw0 + 31 > ib + p.q_start) {  // block touches (or lies above) the diagonal
-      // register r holds query ib + 4hh + c_r with c_r = 8(r/4) + r%4 a compile-time constant:
-      // masked iff key > query + q_start  <=>  key - q_start - ib - 4hh > c_r
-      const int t = key - p.q_start - ib - 4 * hh;
+    if ((p.causal && kw0 + 31 > ib + p.q_start) || ib + 32 > p.Sq) {  // block touches the diagonal or the end of the queries
+      // register r holds query ib + 4hh + c_r with c_r = 8(r/4) + r%4 a compile-time constant.
+      // masked iff key > query + q_start  <=>  c_r < key - q_start - ib - 4hh,   or query >= Sq
+      const int t = p.causal ? key - p.q_start - ib - 4 * hh : -1;
+      const int u = p.Sq - ib - 4 * hh;
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        if (t > 8 * (r >> 2) + (r & 3)) s[r] = -INFINITY;
+      for (int r = 0; r < 16; ++r) {
+        const int c = 8 * (r >> 2) + (r & 3);
+        if (c < t || c >= u) s[r] = -INFINITY;
+      }
     }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -472,37 +433,37 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     }
     const bf16x8 p0 = pack_c_half(s, 0), p1 = pack_c_half(s, 1);
     const bf16x8 ds0 = pack_c_half(dpv, 0), ds1 = pack_c_half(dpv, 1);
-    if (next_rm) request_rowmajor(next_rm, next_qb);
+    if (more) request_rowmajor(next_rm, next_qb);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       dvacc[mb] = mfma32(dT[mb][0], p0, dvacc[mb]);
       dkacc[mb] = mfma32(qT[mb][0], ds0, dkacc[mb]);
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
       dvacc[mb] = mfma32(dT[mb][1], p1, dvacc[mb]);
       dkacc[mb] = mfma32(qT[mb][1], ds1, dkacc[mb]);
     }
   };
 
-  // The loads left in flight across the loop must be the YOUNGEST vector-memory operations: every wait
-  // for an older load (the stationary operands above) would otherwise also drain them in each iteration.
+  // ---- pipeline start-up (see the dQ kernel)
   drain_vector_loads();
-  if (n_it > 2) tile_load(2);
+  if (n_it > 0) issue_tile(0);
+  if (n_it > 1) issue_tile(1);
+  if (n_it > 2) issue_tile(2);
+  if (n_it > 2) wait_vmcnt<kLoadsPerTile>(); else wait_vmcnt<0>();
   __syncthreads();
-  if (n_it > 0) request_rowmajor(rm_base, 0);
+  if (n_it > 0) request_rowmajor(rm_lane, 0);
   int stage = 0;
   for (int it = 0; it < n_it; ++it) {
     const int nstage = stage == kStages - 1 ? 0 : stage + 1;
     const int hq = it / n_vis;
     const int i0 = (qt_start + it - hq * n_vis) * kBK;
-    const char* rm = rm_base + stage * kStageBytes;
-    const char* tr = tr_base + stage * kStageBytes;
-    const float* st = st_base + stage * 128;
-    const char* rm_next = it + 1 < n_it ? rm_base + nstage * kStageBytes : nullptr;
-    step(rm, tr, st, 0, i0, rm, 1);
-    step(rm, tr, st, 1, i0 + 32, rm_next, 0);
-    if (it + 2 < n_it) {
-      tile_store(nstage == kStages - 1 ? 0 : nstage + 1);
-      if (it + 3 < n_it) tile_load(it + 3);
-    }
+    const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
+    const uint32_t st = st_lane + stage * 512;
+    step(tr, st, 0, i0, true, rm, 1);
+    step(tr, st, 1, i0 + 32, it + 1 < n_it, rm_lane + nstage * kStageBytes, 0);
+    if (it + 3 < n_it) { issue_tile(it + 3); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
     __syncthreads();
     stage = nstage;
   }

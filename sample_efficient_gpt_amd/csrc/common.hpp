@@ -14,7 +14,8 @@ constexpr float kLn2 = 0.6931471805599453f;
 // Everything a kernel needs: the caller's params by value plus the carved-up workspace.
 struct KArgs {
   segpt_attn_params p;
-  float* delta;       // [B,H,Sq] fp32: rowsum(dO_eff * o)
+  float* delta;       // [B,H,Sq] fp32: rowsum(dO_eff * o)  (fp32 path) / its NEGATIVE (bf16 path: MFMA C operand)
+  float* nlse2;       // [B,H,Sq] fp32: -lse*log2(e)                 (bf16 path only: MFMA C operand)
   void* do_eff;       // [B,H,Sq,D] dtype, contiguous: gate-scaled dO (only when gated)
   uint16_t* qhat;     // [B,H,Sq,D]   bf16: sm_scale*log2e * a_i q_i * g_q*g_k   (bf16 path only)
   uint16_t* khat;     // [B,Hkv,Sk,D] bf16: b_j k_j                               (bf16 path only)

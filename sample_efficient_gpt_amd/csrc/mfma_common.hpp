@@ -167,6 +167,99 @@ __device__ __forceinline__ bf16x8 frag_tr_at(const char* base, int cb, int s) {
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Swizzled, unpadded LDS tiles filled by direct global->LDS loads (global_load_lds_dwordx4: every lane
+// names its own 16 global bytes, the wave's 64 x 16 B land contiguously at a wave-uniform LDS address).
+// Tile = 64 rows of kRB = 2*D bytes; the 16-byte chunk c of row r is stored at chunk position c ^ (r & 7),
+// which keeps both the row-major b128 fragment reads and the transposing b64 reads free of bank conflicts
+// without padding (padding would break the contiguity the direct loads need).
+template <int D>
+struct Swz {
+  static constexpr int kRB = 2 * D;                     // bytes per row
+  static constexpr int kTileBytes = kBK * kRB;          // 8 KB (D=64) / 16 KB (D=128)
+  static constexpr int kChunks = kRB / 16;              // chunks per row
+  static constexpr int kRowsPerInst = 1024 / kRB;       // rows one wave-wide load covers
+  static constexpr int kPasses = kTileBytes / 1024 / 4; // wave-wide loads per wave per tile (4 waves)
+};
+
+// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt = {imm[15:14], imm[3:0]}, expcnt / lgkmcnt left at max)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
+}
+
+// LDS is addressed by 32-bit byte addresses below (integers, so that the XOR swizzle is plain arithmetic)
+typedef __attribute__((address_space(3))) char* lds_char_ptr;
+__device__ __forceinline__ uint32_t lds_addr_of(const void* shared_obj) {
+  return (uint32_t)(uintptr_t)(lds_char_ptr)shared_obj;
+}
+// The two direct loads are written as inline assembly on purpose: the compiler treats the builtin form
+// as an LDS write of unknown extent and drains every outstanding vector load (s_waitcnt vmcnt(0)) before
+// each barrier and before issuing further ones, which would serialise the whole prefetch pipeline.
+// Completion is tracked by hand instead: wait_vmcnt<N>() followed by __syncthreads() publishes a stage.
+// (Hidden loads only make the compiler's own vmcnt waits conservative, never too weak: the counter
+// retires in order.)
+__device__ __forceinline__ void gload_lds16(const void* gsrc, uint32_t lds_dst_wave_uniform) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gsrc), "s"(lds_dst_wave_uniform)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void gload_lds4(const void* gsrc, uint32_t lds_dst_wave_uniform) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off"
+               :
+               : "v"(gsrc), "s"(lds_dst_wave_uniform)
+               : "memory", "m0");
+}
+__device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
+  return *(const __attribute__((address_space(3))) u32x4*)addr;
+}
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4 lds_read_f4(uint32_t addr) {
+  return *(const __attribute__((address_space(3))) f32x4*)addr;
+}
+
+// Which (row, global chunk) a lane fetches for the wave-wide load number `wave` of a tile (later passes add
+// 4*kRowsPerInst rows, a multiple of 8, so the swizzle term does not change): returns row in .x, byte column in .y
+template <int D>
+__device__ __forceinline__ int2 swz_src(int lane, int wave) {
+  const int row = wave * Swz<D>::kRowsPerInst + lane / Swz<D>::kChunks;
+  const int c = (lane % Swz<D>::kChunks) ^ (row & 7);
+  return make_int2(row, c * 16);
+}
+// Per-lane byte offset (within a tile) of the row-major fragment of k-step 0, row block 0; k-step ks is
+// this offset XOR (ks << 5), row block rb adds 32*kRB.
+template <int D>
+__device__ __forceinline__ int swz_off_rm(int lane) {
+  const int ln = lane & 31, hh = lane >> 5;
+  return ln * Swz<D>::kRB + ((hh ^ (ln & 7)) << 4);
+}
+// Per-lane byte offset of the transposed fragment of column block 0, row step 0 (first of its two
+// 8-byte reads; the second is 8 rows further): column block cb is this offset XOR (cb << 6), row step s
+// adds 16*s*kRB.
+template <int D>
+__device__ __forceinline__ int swz_off_tr(int lane) {
+  const int r = lane & 15, g1 = (lane >> 4) & 1, hh = lane >> 5;
+  const int row = 4 * hh + (r >> 2);          // row & 7 == row
+  const int c = 2 * g1 + ((r & 3) >> 1);      // chunk within the 64-byte column block
+  return row * Swz<D>::kRB + ((c ^ row) << 4) + ((r & 1) << 3);
+}
+template <int D>
+__device__ __forceinline__ bf16x8 swz_frag_rm(uint32_t tile_plus_lane_off, int rb, int ks) {
+  return as_bf16x8(lds_read16((tile_plus_lane_off ^ (uint32_t)(ks << 5)) + rb * 32 * Swz<D>::kRB));
+}
+template <int D>
+__device__ __forceinline__ bf16x8 swz_frag_tr(uint32_t tile_plus_lane_off, int cb, int s) {
+  const uint32_t p = (tile_plus_lane_off ^ (uint32_t)(cb << 6)) + 16 * s * Swz<D>::kRB;
+  typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 8 * Swz<D>::kRB));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
 template <int N>
 using IC = std::integral_constant<int, N>;
 
