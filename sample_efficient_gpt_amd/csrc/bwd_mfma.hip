@@ -107,6 +107,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   constexpr int kLoadsPerTile = 2 * Z::kPasses;  // per wave
   const segpt_attn_params& p = a.p;
   __shared__ __attribute__((aligned(1024))) char lds[kStages * kStageBytes];
+  __shared__ __attribute__((aligned(16))) float gsm[D];       // g_q * g_k, read as float4 slices
+  __shared__ __attribute__((aligned(16))) float red4[4 * D];  // per-wave column sums of the dg partial
   static_assert(kStages * kStageBytes >= 128 * (D + 1) * 4, "LDS reuse for the dg partial");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -139,6 +141,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   };
 
   // ---- query-row prologue: alpha, Qhat, delta, gate; B operands stay in registers
+  if (tid < D) gsm[tid] = gprod_at(p, tid);
+  __syncthreads();
   bf16x8 qreg[KS], doreg[KS];
   float alpha, delta;
   {
@@ -170,12 +174,13 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
+      const float4 ga = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh);
+      const float4 gb = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh + 4);
       u32x4 w;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int d = 16 * ks + 8 * hh + 2 * i;
-        w[i] = pack_bf16x2(bf16lo(qraw[ks][i]) * f * gprod_at(p, d), bf16hi(qraw[ks][i]) * f * gprod_at(p, d + 1));
-      }
+      w[0] = pack_bf16x2(bf16lo(qraw[ks][0]) * f * ga.x, bf16hi(qraw[ks][0]) * f * ga.y);
+      w[1] = pack_bf16x2(bf16lo(qraw[ks][1]) * f * ga.z, bf16hi(qraw[ks][1]) * f * ga.w);
+      w[2] = pack_bf16x2(bf16lo(qraw[ks][2]) * f * gb.x, bf16hi(qraw[ks][2]) * f * gb.y);
+      w[3] = pack_bf16x2(bf16lo(qraw[ks][3]) * f * gb.z, bf16hi(qraw[ks][3]) * f * gb.w);
       qreg[ks] = as_bf16x8(w);
       if (live) *reinterpret_cast<u32x4*>(a.qhat + ridx * D + 16 * ks + 8 * hh) = w;
       if (p.gate.ptr) {
@@ -278,12 +283,18 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   for (int mb = 0; mb < MB; ++mb) {
     load_ct_block(qp, mb, hh, qv[mb]);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int d = 32 * mb + 8 * (r >> 2) + 4 * hh + (r & 3);
-      const float t = acc[mb][r] * p.sm_scale;                 // sm_scale * T
-      red[(wave * 32 + ln) * (D + 1) + d] = live ? t * alpha * qv[mb][r] : 0.f;  // dg contribution of this row
-      acc[mb][r] = t * gprod_at(p, d);                         // u = dL/d(a q)
-      dot += acc[mb][r] * qv[mb][r];
+    for (int c = 0; c < 4; ++c) {
+      const int d0 = 32 * mb + 8 * c + 4 * hh;
+      const float4 g4 = *reinterpret_cast<const float4*>(gsm + d0);
+      const float gv[4] = {g4.x, g4.y, g4.z, g4.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 4 * c + i;
+        const float t = acc[mb][r] * p.sm_scale;                 // sm_scale * T
+        red[(wave * 32 + ln) * (D + 1) + d0 + i] = live ? t * alpha * qv[mb][r] : 0.f;  // dg contribution of this row
+        acc[mb][r] = t * gv[i];                                  // u = dL/d(a q)
+        dot += acc[mb][r] * qv[mb][r];
+      }
     }
   }
   dot = half_sum(dot);
@@ -296,13 +307,17 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     for (int r = 0; r < 16; ++r) val[r] = alpha * acc[mb][r] - a3 * qv[mb][r];
     store_ct_block(op, mb, hh, live, val);
   }
-  // workgroup partial of dg: column sums over the 128 (wave, lane%32) rows
+  // workgroup partial of dg: column sums over the 128 (wave, lane%32) rows, in two levels so that all
+  // 256 threads share the LDS reads (fixed order: deterministic)
   __syncthreads();
-  if (tid < D) {
+  for (int col = tid & 63; col < D; col += 64) {
     float t = 0.f;
-    for (int x = 0; x < 128; ++x) t += red[x * (D + 1) + tid];
-    a.dg_part[(int64_t)blockIdx.x * D + tid] = t;
+#pragma unroll 8
+    for (int x = 0; x < 32; ++x) t += red[(wave * 32 + x) * (D + 1) + col];
+    red4[wave * D + col] = t;
   }
+  __syncthreads();
+  if (tid < D) a.dg_part[(int64_t)blockIdx.x * D + tid] = (red4[tid] + red4[D + tid]) + (red4[2 * D + tid] + red4[3 * D + tid]);
 }
 
 // ============================================================================================ dK, dV

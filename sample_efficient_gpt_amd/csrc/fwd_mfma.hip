@@ -47,6 +47,7 @@ __global__ __launch_bounds__(kThreadsM, 2) void fwd_bf16_kernel(KArgs a) {
   constexpr int MB = D / 32;  // 32-row blocks of O^T
   const segpt_attn_params& p = a.p;
   __shared__ __attribute__((aligned(16))) uint16_t lds[2 * 2 * T::kElems];
+  __shared__ __attribute__((aligned(16))) float gsm[D];  // sm_scale*log2e * g_q * g_k, read as float4 slices
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, hh = lane >> 5;
@@ -62,6 +63,13 @@ __global__ __launch_bounds__(kThreadsM, 2) void fwd_bf16_kernel(KArgs a) {
   const bool bounded = logit_bound(p, lane) <= kNoMaxBound;  // wave-uniform
 
   // ---- Qhat registers: B operands of S^T, [nb][ks]
+  if (tid < D) {
+    float gp = p.gq_numel == 1 ? p.g_q[0] : p.g_q[tid];
+    if (p.gk_numel == 1) gp *= p.g_k[0];
+    else if (p.gk_numel > 1) gp *= p.g_k[tid];
+    gsm[tid] = gp * p.sm_scale * kLog2e;
+  }
+  __syncthreads();
   bf16x8 qreg[NQB][KS];
 #pragma unroll
   for (int nb = 0; nb < NQB; ++nb) {
@@ -75,19 +83,16 @@ __global__ __launch_bounds__(kThreadsM, 2) void fwd_bf16_kernel(KArgs a) {
       ss += sumsq8(raw[ks]);
     }
     ss = half_sum(ss);
-    const float alpha = fast_rsq(ss * (1.0f / D) + p.eps) * p.sm_scale * kLog2e;
+    const float alpha = fast_rsq(ss * (1.0f / D) + p.eps);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
+      const float4 ga = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh);
+      const float4 gb = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh + 4);
       u32x4 w;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int d = 16 * ks + 8 * hh + 2 * i;
-        float g0 = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
-        float g1 = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d + 1];
-        if (p.gk_numel == 1) { g0 *= p.g_k[0]; g1 *= p.g_k[0]; }
-        else if (p.gk_numel > 1) { g0 *= p.g_k[d]; g1 *= p.g_k[d + 1]; }
-        w[i] = pack_bf16x2(bf16lo(raw[ks][i]) * alpha * g0, bf16hi(raw[ks][i]) * alpha * g1);
-      }
+      w[0] = pack_bf16x2(bf16lo(raw[ks][0]) * alpha * ga.x, bf16hi(raw[ks][0]) * alpha * ga.y);
+      w[1] = pack_bf16x2(bf16lo(raw[ks][1]) * alpha * ga.z, bf16hi(raw[ks][1]) * alpha * ga.w);
+      w[2] = pack_bf16x2(bf16lo(raw[ks][2]) * alpha * gb.x, bf16hi(raw[ks][2]) * alpha * gb.y);
+      w[3] = pack_bf16x2(bf16lo(raw[ks][3]) * alpha * gb.z, bf16hi(raw[ks][3]) * alpha * gb.w);
       qreg[nb][ks] = as_bf16x8(w);
     }
   }
