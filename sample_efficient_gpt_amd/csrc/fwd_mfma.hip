@@ -40,7 +40,13 @@ constexpr float kNoMaxBound = 64.f;   // |S2| below this: P in [2^-64, 2^64], su
 constexpr float kLazyThresh = 16.f;   // general path: the subtracted reference is raised only when exceeded by 2^16
 
 template <int D, int NQB, bool VR>
-__global__ __launch_bounds__(kThreadsM, 2) void fwd_bf16_kernel(KArgs a) {
+#ifndef SEGPT_FWD_OCC
+#define SEGPT_FWD_OCC 2
+#endif
+#ifndef SEGPT_FWD_NQB
+#define SEGPT_FWD_NQB 2
+#endif
+__global__ __launch_bounds__(kThreadsM, SEGPT_FWD_OCC) void fwd_bf16_kernel(KArgs a) {
   using T = Tile<D>;
   constexpr int BQ = FwdCfg<D, NQB>::kBQ;
   constexpr int KS = D / 16;  // contraction steps of QK^T
@@ -251,7 +257,7 @@ int launch_fwd_t(const KArgs& a, hipStream_t st) {
 }  // namespace
 
 int launch_fwd_bf16(const KArgs& a, hipStream_t st) {
-  if (a.p.D == 64) return launch_fwd_t<64, 2>(a, st);
+  if (a.p.D == 64) return launch_fwd_t<64, SEGPT_FWD_NQB>(a, st);
   if (a.p.D == 128) return launch_fwd_t<128, 1>(a, st);
   return (int)hipErrorInvalidValue;
 }

@@ -170,9 +170,14 @@ __device__ __forceinline__ bf16x8 frag_tr_at(const char* base, int cb, int s) {
 // ---------------------------------------------------------------------------------------------------
 // Swizzled, unpadded LDS tiles filled by direct global->LDS loads (global_load_lds_dwordx4: every lane
 // names its own 16 global bytes, the wave's 64 x 16 B land contiguously at a wave-uniform LDS address).
-// Tile = 64 rows of kRB = 2*D bytes; the 16-byte chunk c of row r is stored at chunk position c ^ (r & 7),
-// which keeps both the row-major b128 fragment reads and the transposing b64 reads free of bank conflicts
-// without padding (padding would break the contiguity the direct loads need).
+// Tile = 64 rows of kRB = 2*D bytes; the 16-byte chunk c of row r is stored at chunk position c ^ f(r).
+// LDS has 64 banks of 4 bytes; a ds_read_b128 is served 16 lanes at a time, and the 16 lanes of a row-major
+// fragment read sit in 16 consecutive rows at one logical chunk, so f must spread rows that share banks
+// (every second row at D=64, every row at D=128) over distinct chunk positions; the transposing b64 reads
+// touch 4 rows x 32 bytes per 16 lanes and want the rows of a pair two apart in different chunk pairs.
+//   D = 64  (8 chunks / row):   f(r) = (r >> 1) & 7
+//   D = 128 (16 chunks / row):  f(r) = ((r & 3) << 2) | ((r >> 2) & 3)
+// Both depend on r mod 16 only and satisfy f(r + 8) = f(r) ^ kHiXorChunks for r < 8.
 template <int D>
 struct Swz {
   static constexpr int kRB = 2 * D;                     // bytes per row
@@ -180,6 +185,11 @@ struct Swz {
   static constexpr int kChunks = kRB / 16;              // chunks per row
   static constexpr int kRowsPerInst = 1024 / kRB;       // rows one wave-wide load covers
   static constexpr int kPasses = kTileBytes / 1024 / 4; // wave-wide loads per wave per tile (4 waves)
+  static constexpr int kHiXor = (D == 64 ? 4 : 2) << 4; // byte XOR between the swizzle terms of rows r and r+8
+  static __device__ __forceinline__ int f(int row) {
+    return D == 64 ? ((row >> 1) & 7) : (((row & 3) << 2) | ((row >> 2) & 3));
+  }
+  static_assert(D == 64 || D == 128, "swizzle is defined for 128- and 256-byte rows");
 };
 
 // s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt = {imm[15:14], imm[3:0]}, expcnt / lgkmcnt left at max)
@@ -221,11 +231,11 @@ __device__ __forceinline__ f32x4 lds_read_f4(uint32_t addr) {
 }
 
 // Which (row, global chunk) a lane fetches for the wave-wide load number `wave` of a tile (later passes add
-// 4*kRowsPerInst rows, a multiple of 8, so the swizzle term does not change): returns row in .x, byte column in .y
+// 4*kRowsPerInst rows, a multiple of 16, so the swizzle term does not change): returns row in .x, byte column in .y
 template <int D>
 __device__ __forceinline__ int2 swz_src(int lane, int wave) {
   const int row = wave * Swz<D>::kRowsPerInst + lane / Swz<D>::kChunks;
-  const int c = (lane % Swz<D>::kChunks) ^ (row & 7);
+  const int c = (lane % Swz<D>::kChunks) ^ Swz<D>::f(row);
   return make_int2(row, c * 16);
 }
 // Per-lane byte offset (within a tile) of the row-major fragment of k-step 0, row block 0; k-step ks is
@@ -233,17 +243,17 @@ __device__ __forceinline__ int2 swz_src(int lane, int wave) {
 template <int D>
 __device__ __forceinline__ int swz_off_rm(int lane) {
   const int ln = lane & 31, hh = lane >> 5;
-  return ln * Swz<D>::kRB + ((hh ^ (ln & 7)) << 4);
+  return ln * Swz<D>::kRB + ((hh ^ Swz<D>::f(ln)) << 4);
 }
 // Per-lane byte offset of the transposed fragment of column block 0, row step 0 (first of its two
-// 8-byte reads; the second is 8 rows further): column block cb is this offset XOR (cb << 6), row step s
-// adds 16*s*kRB.
+// 8-byte reads; the second is 8 rows further, which also flips kHiXor in the swizzle term): column block
+// cb is this offset XOR (cb << 6), row step s adds 16*s*kRB.
 template <int D>
 __device__ __forceinline__ int swz_off_tr(int lane) {
   const int r = lane & 15, g1 = (lane >> 4) & 1, hh = lane >> 5;
-  const int row = 4 * hh + (r >> 2);          // row & 7 == row
+  const int row = 4 * hh + (r >> 2);          // 0..7
   const int c = 2 * g1 + ((r & 3) >> 1);      // chunk within the 64-byte column block
-  return row * Swz<D>::kRB + ((c ^ row) << 4) + ((r & 1) << 3);
+  return row * Swz<D>::kRB + ((c ^ Swz<D>::f(row)) << 4) + ((r & 1) << 3);
 }
 template <int D>
 __device__ __forceinline__ bf16x8 swz_frag_rm(uint32_t tile_plus_lane_off, int rb, int ks) {
@@ -252,9 +262,10 @@ __device__ __forceinline__ bf16x8 swz_frag_rm(uint32_t tile_plus_lane_off, int r
 template <int D>
 __device__ __forceinline__ bf16x8 swz_frag_tr(uint32_t tile_plus_lane_off, int cb, int s) {
   const uint32_t p = (tile_plus_lane_off ^ (uint32_t)(cb << 6)) + 16 * s * Swz<D>::kRB;
+  const uint32_t q = (tile_plus_lane_off ^ (uint32_t)((cb << 6) ^ Swz<D>::kHiXor)) + (16 * s + 8) * Swz<D>::kRB;
   typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
   s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
-  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 8 * Swz<D>::kRB));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(q));
   typedef short s16x8 __attribute__((ext_vector_type(8)));
   s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   return __builtin_bit_cast(bf16x8, v);
