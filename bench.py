@@ -3,13 +3,14 @@
 
 A step = one forward + one backward of the attention op over one batch of synthetic input, already
 resident in HBM, enqueued through the C ABI (segpt_attn_fwd + segpt_attn_bwd on torch's current
-stream).  Prints ONE JSON line:
+stream; the backward is handed the forward's key/value workspace, as the autograd function does, so the
+key normalisation runs once per step).  Prints ONE JSON line:
 
   value      whole-step algorithmic TFLOP/s: (2 + 5) * B*H*S^2*D / step time (causal FlashAttention
              convention; norm/softmax/gate/mix work and recomputation are not credited)
   roofline   the slowest kernel of the step: its credited FLOPs / its average duration, measured
              with HIP events recorded on the launch stream between the stages while the same K steps
-             are replayed stage by stage (segpt_attn_bwd_stage), vs the MI355X dense bf16 MFMA peak
+             are replayed stage by stage (segpt_attn_fwd_stage / segpt_attn_bwd_stage), vs the MI355X dense bf16 MFMA peak
   cpu_baseline  the CPU restatement of the reference's live path (fp32 RMS-normalise ->
              scaled_dot_product_attention(is_causal) -> autograd backward) timed on this host on a
              bounded sample of the same workload
@@ -95,20 +96,22 @@ def main():
     torch.cuda.set_device(dev)
     x = make_inputs(c, device=dev)
     plan = AttnPlan(x, eps=c.eps, sm_scale=c.sm_scale, gate_scale=c.gate_scale, backward=c.backward)
-    names = ["fwd"] + (["bwd_pre", "bwd_dq", "bwd_dkdv", "bwd_reduce"] if c.backward else [])
+    names = ["kv_prep", "fwd"] + (["bwd_dq", "bwd_dkdv", "bwd_reduce"] if c.backward else [])
 
-    def step_plain():  # the product's two entry points
+    def step_plain():  # the product's two entry points; the backward reuses the forward's normalised keys
         plan.forward()
         if c.backward:
-            plan.backward()
+            plan.backward(kv_prepared=True)
 
     def step_staged(events):  # the same launches, one stage at a time, with an event between them
         events[0].record()
-        plan.forward()
+        plan.forward_stage(0)
         events[1].record()
+        plan.forward_stage(1)
+        events[2].record()
         if c.backward:
-            for s in range(4):
-                plan.backward_stage(s)
+            for s in (1, 2, 3):  # stage 0 (the key/value pre-pass) is skipped: kv_prepared
+                plan.backward_stage(s, kv_prepared=True)
                 events[2 + s].record()
 
     for _ in range(args.warmup):
@@ -143,7 +146,7 @@ def main():
     elem = 2
     hbm_bytes = {  # algorithmic bytes of the HBM-bound helpers
         # K in, Khat out (+ v, v_first in, V' out with a value residual)
-        "bwd_pre": c.B * c.Hkv * c.S * c.D * elem * (5 if c.extras else 2),
+        "kv_prep": c.B * c.Hkv * c.S * c.D * elem * (5 if c.extras else 2),
     }
     kernels = {}
     for n in names:

@@ -58,8 +58,25 @@ extern "C" {
 #define SEGPT_E_ALIGN -10      /* a base pointer is not 16-byte aligned                     */
 #define SEGPT_E_STAGE -11      /* unknown stage passed to segpt_attn_bwd_stage              */
 
+/* segpt_attn_params.flags */
+#define SEGPT_FLAG_KV_PREPARED 1 /* kv_workspace already holds what the key/value pre-pass writes for these k, v,
+                                    v_first, vr_coef and eps (e.g. segpt_attn_fwd just ran on it): skip the pre-pass */
+
+#define SEGPT_FLAG_RUNNING_MAX 2 /* bf16 forward: always subtract a running row maximum before exp2, also when the
+                                    QK-norm bound on the logits (sm_scale*D*max|g_q g_k|) would allow the raw
+                                    exponent; same results up to rounding, slower */
+
+/* which scratch buffer segpt_attn_workspace_bytes() sizes */
+#define SEGPT_WS_KV 0  /* kv_workspace: bf16 copies of the normalised keys (and mixed values); forward AND backward */
+#define SEGPT_WS_BWD 1 /* workspace: per-row statistics, normalised queries, partial sums; backward only            */
+
+/* the two stages segpt_attn_fwd() runs, in this order */
+#define SEGPT_FWD_STAGE_PRE 0  /* bf16: key/value pre-pass (skipped with SEGPT_FLAG_KV_PREPARED); fp32: nothing */
+#define SEGPT_FWD_STAGE_ATTN 1 /* the attention kernel: writes o and lse                                         */
+
 /* the four stages segpt_attn_bwd() runs, in this order */
-#define SEGPT_BWD_STAGE_PRE 0    /* bf16: normalised Khat (and V' = c1 v + c2 v_first) into the workspace;
+#define SEGPT_BWD_STAGE_PRE 0    /* bf16: key/value pre-pass (skipped with SEGPT_FLAG_KV_PREPARED): normalised
+                                    Khat (and V' = c1 v + c2 v_first) into kv_workspace;
                                     fp32: delta = rowsum(dY*Y), dgate and the gate-scaled dO            */
 #define SEGPT_BWD_STAGE_DQ 1     /* dQ and the per-workgroup partials of the scale gradient; on the bf16
                                     path also delta, dgate, Qhat and the gate-scaled dO for stage 2      */
@@ -89,7 +106,7 @@ typedef struct segpt_attn_params {
   int32_t gq_numel; /* 1 (scalar gain, attention.py:41) or D */
   int32_t gk_numel; /* 0 (no k scale), 1 or D */
   float eps, sm_scale, gate_scale;
-  int32_t reserved0;
+  int32_t flags; /* SEGPT_FLAG_* */
 
   /* forward operands */
   segpt_tensor4 q;       /* [B,H,Sq,D]   in  */
@@ -114,8 +131,13 @@ typedef struct segpt_attn_params {
   float* dg_k;            /* [gk_numel] fp32 out, required iff g_k */
   float* dvr_coef;        /* [2] fp32 out, required iff vr_coef */
 
-  void* workspace; /* >= segpt_attn_workspace_bytes(), 256 B aligned; contents undefined on entry */
+  void* workspace; /* backward only: >= segpt_attn_workspace_bytes(p, SEGPT_WS_BWD), 256 B aligned; contents
+                      undefined on entry */
   size_t workspace_bytes;
+  void* kv_workspace; /* bf16 forward and backward: >= segpt_attn_workspace_bytes(p, SEGPT_WS_KV), 256 B aligned.
+                         Written by the key/value pre-pass of either call; a backward that gets the buffer its
+                         forward used may set SEGPT_FLAG_KV_PREPARED.  Ignored (may be NULL) for fp32. */
+  size_t kv_workspace_bytes;
 } segpt_attn_params;
 
 /* ABI revision of the loaded library (compare with SEGPT_ABI_VERSION). No reference counterpart. */
@@ -125,13 +147,13 @@ int segpt_abi_version(void);
  * Replaces the Python AssertionErrors of triton_flash_attn_qknorm.py:273-276. */
 const char* segpt_strerror(int code);
 
-/* Bytes of device scratch the call needs (0 is possible for forward). Validates nothing but
- * sizes; returns 0 for invalid params (the launch call will report the error).
+/* Bytes of device scratch of kind `which` (SEGPT_WS_*) these params need (0 is possible). Validates
+ * nothing but sizes; returns 0 for invalid params (the launch call will report the error).
  * Replaces the in-op allocations of triton_flash_attn_qknorm.py:286-287 / :320-323: the caller
  * allocates. */
-size_t segpt_attn_workspace_bytes(const segpt_attn_params* p, int is_bwd);
+size_t segpt_attn_workspace_bytes(const segpt_attn_params* p, int which);
 
-/* Forward: writes o (y) and lse.  Replaces the launch
+/* Forward: writes o (y) and lse (bf16: and kv_workspace).  Replaces the launch
  * `flashatt_qknorm_kernel_fwd[grid](...)`, triton_flash_attn_qknorm.py:290-302 (kernel :22-115),
  * and in the live path the normalise + SDPA sequence attention.py:52-80. */
 int segpt_attn_fwd(const segpt_attn_params* p, void* stream);
@@ -146,6 +168,10 @@ int segpt_attn_bwd(const segpt_attn_params* p, void* stream);
  * and workspace.  Each stage needs the earlier ones to have run on the same workspace.  No counterpart in the
  * reference (its backward is the single kernel triton_flash_attn_qknorm.py:125-255). */
 int segpt_attn_bwd_stage(const segpt_attn_params* p, int stage, void* stream);
+
+/* The same for the forward: segpt_attn_fwd(p, s) is stages SEGPT_FWD_STAGE_PRE, SEGPT_FWD_STAGE_ATTN in this
+ * order.  No counterpart in the reference (its forward is the single kernel triton_flash_attn_qknorm.py:22-115). */
+int segpt_attn_fwd_stage(const segpt_attn_params* p, int stage, void* stream);
 
 #ifdef __cplusplus
 }

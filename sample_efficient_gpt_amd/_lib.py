@@ -15,6 +15,11 @@ LIB_PATH = os.path.join(PKG_DIR, "libsegpt_attn.so")
 SEGPT_ABI_VERSION = 1
 SEGPT_DTYPE_BF16 = 0
 SEGPT_DTYPE_FP32 = 1
+SEGPT_FLAG_KV_PREPARED = 1
+SEGPT_FLAG_RUNNING_MAX = 2
+SEGPT_WS_KV = 0
+SEGPT_WS_BWD = 1
+FWD_STAGES = ("pre", "attn")  # SEGPT_FWD_STAGE_* = index
 BWD_STAGES = ("pre", "dq", "dkdv", "reduce")  # SEGPT_BWD_STAGE_* = index
 
 EXPORTED_SYMBOLS = (
@@ -24,6 +29,7 @@ EXPORTED_SYMBOLS = (
     "segpt_attn_fwd",
     "segpt_attn_bwd",
     "segpt_attn_bwd_stage",
+    "segpt_attn_fwd_stage",
 )
 
 
@@ -45,7 +51,7 @@ class AttnParams(C.Structure):
         ("gq_numel", C.c_int32),
         ("gk_numel", C.c_int32),
         ("eps", C.c_float), ("sm_scale", C.c_float), ("gate_scale", C.c_float),
-        ("reserved0", C.c_int32),
+        ("flags", C.c_int32),
         ("q", Tensor4), ("k", Tensor4), ("v", Tensor4), ("v_first", Tensor4),
         ("gate", Tensor3),
         ("o", Tensor4),
@@ -56,6 +62,8 @@ class AttnParams(C.Structure):
         ("dg_q", C.c_void_p), ("dg_k", C.c_void_p), ("dvr_coef", C.c_void_p),
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
+        ("kv_workspace", C.c_void_p),
+        ("kv_workspace_bytes", C.c_size_t),
     ]
 
 
@@ -95,6 +103,8 @@ def load():
         lib.segpt_attn_bwd.argtypes = [C.POINTER(AttnParams), C.c_void_p]
         lib.segpt_attn_bwd_stage.restype = C.c_int
         lib.segpt_attn_bwd_stage.argtypes = [C.POINTER(AttnParams), C.c_int, C.c_void_p]
+        lib.segpt_attn_fwd_stage.restype = C.c_int
+        lib.segpt_attn_fwd_stage.argtypes = [C.POINTER(AttnParams), C.c_int, C.c_void_p]
         ver = lib.segpt_abi_version()
         if ver != SEGPT_ABI_VERSION:
             raise RuntimeError(f"libsegpt_attn.so ABI version {ver}, binding expects {SEGPT_ABI_VERSION}")
@@ -130,3 +140,11 @@ def t3(t) -> Tensor3:
 
 def ptr(t):
     return None if t is None else t.data_ptr()
+
+
+def alloc_workspace(lib, p, which: int, device):
+    """Allocate (torch, uint8) the scratch buffer of kind `which` for filled params; returns the tensor."""
+    import torch
+
+    nbytes = max(int(lib.segpt_attn_workspace_bytes(p, which)), 256)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)

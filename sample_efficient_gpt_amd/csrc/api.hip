@@ -23,8 +23,23 @@ size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 size_t elem_bytes(const segpt_attn_params& p) { return p.dtype == SEGPT_DTYPE_FP32 ? 4 : 2; }
 
 struct WsLayout {
-  size_t delta, nlse2, do_eff, qhat, khat, vmix, dg_part, dcoef_part, total;
+  size_t delta, nlse2, do_eff, qhat, dg_part, dcoef_part, total;
 };
+struct KvLayout {
+  size_t khat, vmix, total;
+};
+
+// bf16 only: normalised keys and (with a value residual) mixed values, contiguous [B,Hkv,Sk,D]
+KvLayout kv_layout(const segpt_attn_params& p) {
+  KvLayout w{0, 0, 0};
+  if (p.dtype != SEGPT_DTYPE_BF16) return w;
+  const size_t kvrows = (size_t)p.B * p.Hkv * p.Sk;
+  size_t off = align_up(kvrows * p.D * 2);
+  w.vmix = off;
+  if (p.v_first.ptr) off += align_up(kvrows * p.D * 2);
+  w.total = off;
+  return w;
+}
 
 WsLayout bwd_layout(const segpt_attn_params& p) {
   WsLayout w;
@@ -36,15 +51,8 @@ WsLayout bwd_layout(const segpt_attn_params& p) {
   if (p.dtype == SEGPT_DTYPE_BF16) off += align_up(rows * sizeof(float));
   w.do_eff = off;
   if (p.gate.ptr) off += align_up(rows * p.D * elem_bytes(p));
-  w.qhat = w.khat = w.vmix = off;
-  if (p.dtype == SEGPT_DTYPE_BF16) {
-    const size_t kvrows = (size_t)p.B * p.Hkv * p.Sk;
-    off += align_up(rows * p.D * 2);
-    w.khat = off;
-    off += align_up(kvrows * p.D * 2);
-    w.vmix = off;
-    if (p.v_first.ptr) off += align_up(kvrows * p.D * 2);
-  }
+  w.qhat = off;
+  if (p.dtype == SEGPT_DTYPE_BF16) off += align_up(rows * p.D * 2);
   w.dg_part = off;
   off += align_up((size_t)dq_blocks(p) * p.D * sizeof(float));
   w.dcoef_part = off;
@@ -89,7 +97,21 @@ int check_common(const segpt_attn_params* p) {
   if ((rc = check_t4(p->o, *p))) return rc;
   if (p->v_first.ptr && (rc = check_t4(p->v_first, *p))) return rc;
   if (p->gate.ptr && (p->gate.stride_b < 0 || p->gate.stride_s < 0 || p->gate.stride_h < 0)) return SEGPT_E_STRIDE;
+  if (p->dtype == SEGPT_DTYPE_BF16) {
+    if (!p->kv_workspace || p->kv_workspace_bytes < kv_layout(*p).total) return SEGPT_E_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(p->kv_workspace) & 255u) return SEGPT_E_ALIGN;
+  }
   return SEGPT_OK;
+}
+
+// fills the kernel arguments that both directions share
+void bind_kv(KArgs& a) {
+  const segpt_attn_params& p = a.p;
+  if (p.dtype != SEGPT_DTYPE_BF16) return;
+  const KvLayout kv = kv_layout(p);
+  char* ws = reinterpret_cast<char*>(p.kv_workspace);
+  a.khat = reinterpret_cast<uint16_t*>(ws + kv.khat);
+  a.vmix = p.v_first.ptr ? reinterpret_cast<uint16_t*>(ws + kv.vmix) : nullptr;
 }
 
 int check_bwd(const segpt_attn_params* p) {
@@ -132,30 +154,50 @@ const char* segpt_strerror(int code) {
     case SEGPT_E_SHAPE: return "bad shape: sizes must be positive, H divisible by Hkv, scale vectors of 1 or D elements";
     case SEGPT_E_HEAD_DIM: return "unsupported head_dim: bf16 needs D in {64,128}, fp32 D in {32,64,128}";
     case SEGPT_E_STRIDE: return "bad stride: strides must be non-negative multiples of 16 bytes and rows must not overlap";
-    case SEGPT_E_WORKSPACE: return "workspace missing or smaller than segpt_attn_workspace_bytes()";
+    case SEGPT_E_WORKSPACE: return "workspace or kv_workspace missing or smaller than segpt_attn_workspace_bytes()";
     case SEGPT_E_EXTRAS: return "inconsistent optional operands (v_first/vr_coef/gate and their gradient slots)";
     case SEGPT_E_QSTART: return "q_start must be >= 0";
     case SEGPT_E_ALIGN: return "a base pointer is not 16-byte aligned (workspace: 256-byte)";
-    case SEGPT_E_STAGE: return "unknown backward stage (expected SEGPT_BWD_STAGE_*)";
+    case SEGPT_E_STAGE: return "unknown stage (expected SEGPT_FWD_STAGE_* / SEGPT_BWD_STAGE_*)";
     default: return code > 0 ? "HIP runtime error raised by a kernel launch" : "unknown segpt error code";
   }
 }
 
-size_t segpt_attn_workspace_bytes(const segpt_attn_params* p, int is_bwd) {
+size_t segpt_attn_workspace_bytes(const segpt_attn_params* p, int which) {
   if (!p || p->struct_bytes != sizeof(segpt_attn_params)) return 0;
   if (p->B <= 0 || p->H <= 0 || p->Hkv <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0) return 0;
-  if (!is_bwd) return 0;
   if (p->dtype == SEGPT_DTYPE_BF16 && p->D != 64 && p->D != 128) return 0;
-  return bwd_layout(*p).total;
+  if (which == SEGPT_WS_KV) return kv_layout(*p).total;
+  if (which == SEGPT_WS_BWD) return bwd_layout(*p).total;
+  return 0;
 }
 
-int segpt_attn_fwd(const segpt_attn_params* p, void* stream) {
+static int fwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi, void* stream) {
   int rc = check_common(p);
   if (rc) return rc;
   KArgs a{};
   a.p = *p;
+  bind_kv(a);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  return p->dtype == SEGPT_DTYPE_FP32 ? launch_fwd_f32(a, st) : launch_fwd_bf16(a, st);
+  const bool f32 = p->dtype == SEGPT_DTYPE_FP32;
+  for (int stage = stage_lo; stage <= stage_hi; ++stage) {
+    switch (stage) {
+      case SEGPT_FWD_STAGE_PRE: rc = (f32 || (p->flags & SEGPT_FLAG_KV_PREPARED)) ? 0 : launch_kv_prep(a, st); break;
+      case SEGPT_FWD_STAGE_ATTN: rc = f32 ? launch_fwd_f32(a, st) : launch_fwd_bf16(a, st); break;
+      default: return SEGPT_E_STAGE;
+    }
+    if (rc) return rc;
+  }
+  return SEGPT_OK;
+}
+
+int segpt_attn_fwd(const segpt_attn_params* p, void* stream) {
+  return fwd_stage_impl(p, SEGPT_FWD_STAGE_PRE, SEGPT_FWD_STAGE_ATTN, stream);
+}
+
+int segpt_attn_fwd_stage(const segpt_attn_params* p, int stage, void* stream) {
+  if (stage < SEGPT_FWD_STAGE_PRE || stage > SEGPT_FWD_STAGE_ATTN) return SEGPT_E_STAGE;
+  return fwd_stage_impl(p, stage, stage, stream);
 }
 
 static int bwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi, void* stream) {
@@ -173,16 +215,17 @@ static int bwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi
   if (p->dtype == SEGPT_DTYPE_BF16) {
     a.nlse2 = reinterpret_cast<float*>(ws + w.nlse2);
     a.qhat = reinterpret_cast<uint16_t*>(ws + w.qhat);
-    a.khat = reinterpret_cast<uint16_t*>(ws + w.khat);
-    a.vmix = p->v_first.ptr ? reinterpret_cast<uint16_t*>(ws + w.vmix) : nullptr;
   }
+  bind_kv(a);
   a.n_dq_blocks = dq_blocks(*p);
   a.n_dkdv_blocks = dkdv_blocks(*p);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool f32 = p->dtype == SEGPT_DTYPE_FP32;
   for (int stage = stage_lo; stage <= stage_hi; ++stage) {
     switch (stage) {
-      case SEGPT_BWD_STAGE_PRE: rc = launch_bwd_pre(a, st); break;
+      case SEGPT_BWD_STAGE_PRE:
+        rc = f32 ? launch_bwd_pre(a, st) : ((p->flags & SEGPT_FLAG_KV_PREPARED) ? 0 : launch_kv_prep(a, st));
+        break;
       case SEGPT_BWD_STAGE_DKDV: rc = f32 ? launch_bwd_dkdv_f32(a, st) : launch_bwd_dkdv_bf16(a, st); break;
       case SEGPT_BWD_STAGE_DQ: rc = f32 ? launch_bwd_dq_f32(a, st) : launch_bwd_dq_bf16(a, st); break;
       case SEGPT_BWD_STAGE_REDUCE: rc = launch_bwd_reduce(a, st); break;

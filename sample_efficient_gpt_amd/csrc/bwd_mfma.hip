@@ -27,64 +27,7 @@ namespace {
 
 constexpr int kBwdRows = 4 * 32;  // rows (queries for dQ, keys for dK/dV) owned by a workgroup
 
-__device__ __forceinline__ float gprod_at(const segpt_attn_params& p, int d) {
-  float g = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
-  if (p.gk_numel == 1) g *= p.g_k[0];
-  else if (p.gk_numel > 1) g *= p.g_k[d];
-  return g;
-}
-
-// store a C tile column block: lane = row of the output tensor, registers = 32 consecutive columns
-// starting at 32*mb, values already scaled.  Lanes l and l^32 exchange halves so that each lane
-// writes 16 contiguous bytes.
-__device__ __forceinline__ void store_ct_block(uint16_t* rowp, int mb, int hh, bool live, const float (&val)[16]) {
-#pragma unroll
-  for (int cc = 0; cc < 2; ++cc) {
-    const uint32_t x0 = pack_bf16x2(val[8 * cc + 0], val[8 * cc + 1]);
-    const uint32_t x1 = pack_bf16x2(val[8 * cc + 2], val[8 * cc + 3]);
-    const uint32_t y0 = pack_bf16x2(val[8 * cc + 4], val[8 * cc + 5]);
-    const uint32_t y1 = pack_bf16x2(val[8 * cc + 6], val[8 * cc + 7]);
-    auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
-    auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-    const u32x4 w = {s0[0], s1[0], s0[1], s1[1]};
-    if (live) *reinterpret_cast<u32x4*>(rowp + 32 * mb + 16 * cc + 8 * hh) = w;
-  }
-}
-
-// raw bf16 values of a tensor row at the 16 columns a lane's C registers of block mb map to
-__device__ __forceinline__ void load_ct_block(const uint16_t* rowp, int mb, int hh, float (&out)[16]) {
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const u32x2 w = *reinterpret_cast<const u32x2*>(rowp + 32 * mb + 8 * c + 4 * hh);
-    out[4 * c + 0] = bf16lo(w[0]); out[4 * c + 1] = bf16hi(w[0]);
-    out[4 * c + 2] = bf16lo(w[1]); out[4 * c + 3] = bf16hi(w[1]);
-  }
-}
-
-__device__ __forceinline__ f32x16 splat16(float x) {
-  f32x16 v;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) v[r] = x;
-  return v;
-}
-
 constexpr int kStages = 4;  // LDS ring of streamed stages (two tiles each): tile t lives in stage t % 4
-
-// Issue the direct global->LDS loads of two [64, D] bf16 tiles (rows row0..row0+63 of two row-major
-// tensors; rows past nrows re-read the last valid row, callers mask them) into one stage.
-//   src_a/src_b: wave-uniform pointers to row `row0` of each tensor; step_*: bytes between rows
-//   dst: LDS byte address of the stage + wave*1024 (wave-uniform); lane_row / lane_col: from swz_src()
-template <int D>
-__device__ __forceinline__ void issue_tile_pair(const char* src_a, uint32_t step_a, const char* src_b, uint32_t step_b,
-                                                int rows_left, uint32_t dst, int lane_row, int lane_col) {
-  using Z = Swz<D>;
-#pragma unroll
-  for (int ps = 0; ps < Z::kPasses; ++ps) {
-    const int row = min(lane_row + ps * 4 * Z::kRowsPerInst, rows_left - 1);
-    gload_lds16(src_a + (uint32_t)row * step_a + lane_col, dst + ps * 4096);
-    gload_lds16(src_b + (uint32_t)row * step_b + lane_col, dst + Z::kTileBytes + ps * 4096);
-  }
-}
 
 // ============================================================================================ dQ
 // Also the producer of the per-query-row quantities the dK/dV kernel streams afterwards: Qhat, -delta,

@@ -18,8 +18,8 @@ struct KArgs {
   float* nlse2;       // [B,H,Sq] fp32: -lse*log2(e)                 (bf16 path only: MFMA C operand)
   void* do_eff;       // [B,H,Sq,D] dtype, contiguous: gate-scaled dO (only when gated)
   uint16_t* qhat;     // [B,H,Sq,D]   bf16: sm_scale*log2e * a_i q_i * g_q*g_k   (bf16 path only)
-  uint16_t* khat;     // [B,Hkv,Sk,D] bf16: b_j k_j                               (bf16 path only)
-  uint16_t* vmix;     // [B,Hkv,Sk,D] bf16: c1 v + c2 v_first (only with a value residual, else NULL)
+  uint16_t* khat;     // [B,Hkv,Sk,D] bf16: b_j k_j                               (bf16 path only; kv_workspace)
+  uint16_t* vmix;     // [B,Hkv,Sk,D] bf16: c1 v + c2 v_first (only with a value residual, else NULL; kv_workspace)
   float* dg_part;     // [n_dq_blocks, D] fp32 partial sums of the combined scale gradient
   float* dcoef_part;  // [n_dkdv_blocks, 2] fp32 partial sums of (dc1, dc2)
   int32_t n_dq_blocks;
@@ -101,7 +101,8 @@ int launch_bwd_dq_f32(const KArgs& a, hipStream_t st);
 int launch_fwd_bf16(const KArgs& a, hipStream_t st);
 int launch_bwd_dkdv_bf16(const KArgs& a, hipStream_t st);
 int launch_bwd_dq_bf16(const KArgs& a, hipStream_t st);
-int launch_bwd_pre(const KArgs& a, hipStream_t st);     // delta, dgate, do_eff
+int launch_bwd_pre(const KArgs& a, hipStream_t st);     // fp32 path: delta, dgate, do_eff
+int launch_kv_prep(const KArgs& a, hipStream_t st);     // bf16 path: Khat (and V') into kv_workspace
 int launch_bwd_reduce(const KArgs& a, hipStream_t st);  // dg_q, dg_k, dvr_coef from the partials
 
 // block counts shared by the workspace carve-up and the launchers

@@ -1,24 +1,18 @@
-// bf16 forward: causal GQA flash attention with the QK RMS-norm fused into the tile loads.
+// bf16 forward: causal GQA flash attention on the normalised keys of the key/value pre-pass.
 //
-// Workgroup = 4 waves (two workgroups share a CU so that one's softmax overlaps the other's MFMAs);
-// wave w owns NQB blocks of 32 queries.  Scores are produced TRANSPOSED,
+// Workgroup = 4 waves (two workgroups share a CU at head_dim 64 so that one's softmax overlaps the other's
+// MFMAs); wave w owns NQB blocks of 32 queries.  Scores are produced TRANSPOSED,
 //   S^T[key][query] = Khat[key][:] . Qhat[query][:]          (A = Khat tile from LDS, B = Qhat registers)
-// so every lane owns one query column: the online-softmax state (m, l) and the rescale factor are
-// per-lane scalars, row reductions are in-register plus one exchange with lane^32, and the bf16
-// probabilities are already laid out as the B operand of
+// so every lane owns one query column: the softmax state (reference point, row sum) is a per-lane scalar,
+// row reductions are in-register plus one exchange with lane^32, and the bf16 probabilities are already
+// laid out as the B operand of
 //   O^T[d][query] += V'^T[d][key] . P^T[key][query]          (A = transposing LDS read of the V' tile).
-// Qhat = sm_scale*log2(e) * a_i * q_i * g_q * g_k  (both scale vectors live on the query side),
-// Khat = b_j * k_j, V' = c1 v + c2 v_first; all three are formed in fp32 and rounded to bf16 once.
-// K/V tiles (64 keys) are double-buffered in LDS against the global loads of the next tile.
+// Qhat = sm_scale*log2(e) * a_i * q_i * g_q * g_k  (both scale vectors live on the query side) is formed in
+// the prologue; Khat = b_j * k_j and V' = c1 v + c2 v_first are read as written by the pre-pass.
 #include "mfma_common.hpp"
 
 namespace segpt {
 namespace {
-
-template <int D, int NQB>
-struct FwdCfg {
-  static constexpr int kBQ = 4 * 32 * NQB;  // queries per workgroup
-};
 
 // Largest |log2-unit logit| the normalised operands can produce: |Qhat.Khat| <= |Qhat| |Khat| with
 // |Khat| <= sqrt(D) and |Qhat| <= sm_scale*log2e*sqrt(D)*max|g_q g_k|.  When it is small the softmax needs
@@ -39,20 +33,33 @@ __device__ __forceinline__ float logit_bound(const segpt_attn_params& p, int lan
 constexpr float kNoMaxBound = 64.f;   // |S2| below this: P in [2^-64, 2^64], sums stay far inside fp32 range
 constexpr float kLazyThresh = 16.f;   // general path: the subtracted reference is raised only when exceeded by 2^16
 
-template <int D, int NQB, bool VR>
-#ifndef SEGPT_FWD_OCC
-#define SEGPT_FWD_OCC 2
-#endif
-#ifndef SEGPT_FWD_NQB
-#define SEGPT_FWD_NQB 2
-#endif
-__global__ __launch_bounds__(kThreadsM, SEGPT_FWD_OCC) void fwd_bf16_kernel(KArgs a) {
-  using T = Tile<D>;
-  constexpr int BQ = FwdCfg<D, NQB>::kBQ;
-  constexpr int KS = D / 16;  // contraction steps of QK^T
-  constexpr int MB = D / 32;  // 32-row blocks of O^T
+// Khat / V' come from the key/value pre-pass (bf16, contiguous [B,Hkv,Sk,D]) and travel global->LDS
+// directly into a swizzled ring of stages, so the loop holds no staging registers and no normalisation
+// work.  Software pipeline over 32-key blocks n (two per staged tile), one barrier per tile:
+//   B(n)   S^T MFMAs from the row-major Khat fragments requested one block earlier
+//   C(n)   request the transposed V' fragments of block n
+//   D(n)   mask (diagonal blocks only), exp2, bf16 pack, row sums
+//   A(n+1) request the row-major Khat fragments of block n+1 (possibly of the next tile, already landed)
+//   E(n)   O^T += V'^T P^T MFMAs
+template <int D>
+struct FwdShape {
+  static constexpr int kNQB = D == 64 ? 2 : 1;     // 32-query blocks per wave
+  static constexpr int kStages = D == 64 ? 4 : 3;  // LDS: 64 KB (two workgroups per CU) / 96 KB
+  static constexpr int kOcc = D == 64 ? 2 : 1;
+  static constexpr int kBQ = 4 * 32 * kNQB;
+};
+
+template <int D>
+__global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(KArgs a) {
+  using Z = Swz<D>;
+  using F = FwdShape<D>;
+  constexpr int NQB = F::kNQB, BQ = F::kBQ, NS = F::kStages;
+  constexpr int KS = D / 16;
+  constexpr int MB = D / 32;
+  constexpr int kStageBytes = 2 * Z::kTileBytes;
+  constexpr int kLoadsPerTile = 2 * Z::kPasses;  // per wave
   const segpt_attn_params& p = a.p;
-  __shared__ __attribute__((aligned(16))) uint16_t lds[2 * 2 * T::kElems];
+  __shared__ __attribute__((aligned(1024))) char lds[NS * kStageBytes];
   __shared__ __attribute__((aligned(16))) float gsm[D];  // sm_scale*log2e * g_q * g_k, read as float4 slices
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -63,18 +70,26 @@ __global__ __launch_bounds__(kThreadsM, SEGPT_FWD_OCC) void fwd_bf16_kernel(KArg
   const int b = wg.b, g = wg.g, h = wg.g * rep + wg.hh;
   const int q0 = wg.tile * BQ;
   const int qw0 = q0 + wave * 32 * NQB;  // first query of this wave
+  const bool bounded = !(p.flags & SEGPT_FLAG_RUNNING_MAX) && logit_bound(p, lane) <= kNoMaxBound;  // wave-uniform
 
-  float c1 = 1.f, c2 = 0.f;
-  if (VR) { c1 = p.vr_coef[0]; c2 = p.vr_coef[1]; }
-  const bool bounded = logit_bound(p, lane) <= kNoMaxBound;  // wave-uniform
+  int kend = p.Sk;
+  if (p.causal) kend = min(p.Sk, q0 + BQ + p.q_start);
+  const int n_kt = (kend + kBK - 1) / kBK;
+  const char* kbase = reinterpret_cast<const char*>(a.khat + ((int64_t)b * p.Hkv + g) * p.Sk * D);
+  const char* vbase = a.vmix ? reinterpret_cast<const char*>(a.vmix + ((int64_t)b * p.Hkv + g) * p.Sk * D)
+                             : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.v, b, g, 0));
+  const uint32_t kstep = D * 2, vstep = a.vmix ? (uint32_t)D * 2 : (uint32_t)p.v.stride_s * 2;
+
+  const uint32_t lds0 = lds_addr_of(lds);
+  const int2 src = swz_src<D>(lane, wave);
+  const uint32_t wave_dst = lds0 + __builtin_amdgcn_readfirstlane(wave) * 1024;
+  auto issue_tile = [&](int jt) {  // tile jt -> stage jt % NS
+    issue_tile_pair<D>(kbase + (int64_t)jt * kBK * kstep, kstep, vbase + (int64_t)jt * kBK * vstep, vstep,
+                       p.Sk - jt * kBK, wave_dst + (jt % NS) * kStageBytes, src.x, src.y);
+  };
 
   // ---- Qhat registers: B operands of S^T, [nb][ks]
-  if (tid < D) {
-    float gp = p.gq_numel == 1 ? p.g_q[0] : p.g_q[tid];
-    if (p.gk_numel == 1) gp *= p.g_k[0];
-    else if (p.gk_numel > 1) gp *= p.g_k[tid];
-    gsm[tid] = gp * p.sm_scale * kLog2e;
-  }
+  if (tid < D) gsm[tid] = gprod_at(p, tid) * p.sm_scale * kLog2e;
   __syncthreads();
   bf16x8 qreg[NQB][KS];
 #pragma unroll
@@ -107,107 +122,138 @@ __global__ __launch_bounds__(kThreadsM, SEGPT_FWD_OCC) void fwd_bf16_kernel(KArg
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < NQB; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[mb][nb][r] = 0.f;
+    for (int nb = 0; nb < NQB; ++nb) oacc[mb][nb] = splat16(0.f);
   // m_ref: the value subtracted from the logits before exp2 (0 on the bounded path); l_run: this lane's
   // share of the row sum (its half of the keys; halves are added in the epilogue)
   float m_ref[NQB], l_run[NQB];
+  int qlim[NQB];  // last visible key of this lane's query in block nb
 #pragma unroll
-  for (int nb = 0; nb < NQB; ++nb) { m_ref[nb] = bounded ? 0.f : -INFINITY; l_run[nb] = 0.f; }
+  for (int nb = 0; nb < NQB; ++nb) {
+    m_ref[nb] = bounded ? 0.f : -INFINITY;
+    l_run[nb] = 0.f;
+    qlim[nb] = p.causal ? min(qw0 + 32 * nb + ln + p.q_start, p.Sk - 1) : p.Sk - 1;
+  }
 
-  int kend = p.Sk;
-  if (p.causal) kend = min(p.Sk, q0 + BQ + p.q_start);
-  const int n_kt = (kend + kBK - 1) / kBK;
+  // 32-key blocks this wave has to visit (causal: up to the block holding its last query's diagonal)
+  int n_act = (kend + 31) / 32;
+  if (p.causal) n_act = min(n_act, (qw0 + 32 * NQB - 1 + p.q_start) / 32 + 1);
 
-  StageRegs<D> sr;
-  stage_load<D, VR>(p, b, g, 0, sr);
-  stage_store<D, VR>(sr, lds, lds + T::kElems, p.eps, c1, c2);
-  __syncthreads();
-
-  for (int jt = 0; jt < n_kt; ++jt) {
-    const int j0 = jt * kBK;
-    const uint16_t* kt = lds + (jt & 1) * 2 * T::kElems;
-    const uint16_t* vt = kt + T::kElems;
-    const bool more = jt + 1 < n_kt;
-    if (more) stage_load<D, VR>(p, b, g, j0 + kBK, sr);
-
+  const uint32_t rm_lane = lds0 + swz_off_rm<D>(lane);
+  const uint32_t tr_lane = lds0 + swz_off_tr<D>(lane) + Z::kTileBytes;  // V' tile of a stage
+  bf16x8 kf[KS];
+  auto request_rowmajor = [&](uint32_t rm, int kb) {  // kb compile-time at every call site
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const int jb = j0 + 32 * kb;  // first key of this 32-key block
-      // wave-uniform: does this wave see any key of the block?
-      const bool active = jb < p.Sk && (!p.causal || jb <= qw0 + 32 * NQB - 1 + p.q_start);
-      if (active) {
-        f32x16 s[NQB];
+    for (int ks = 0; ks < KS; ++ks) kf[ks] = swz_frag_rm<D>(rm, kb, ks);
+  };
+  // One 32-key block.  MASKED / BOUNDED are compile-time so that a whole block is one straight-line
+  // scheduling region (a branch in the middle would keep the compiler from interleaving the exp2 work with
+  // the neighbouring MFMAs and LDS reads).
+  auto step = [&](auto masked_c, auto bounded_c, uint32_t tr, int kb, int jb, bool more, uint32_t next_rm, int next_kb) {
+    constexpr bool MASKED = decltype(masked_c)::value != 0, BOUNDED = decltype(bounded_c)::value != 0;
+    f32x16 s[NQB];
 #pragma unroll
-        for (int nb = 0; nb < NQB; ++nb)
+    for (int nb = 0; nb < NQB; ++nb) s[nb] = splat16(0.f);
 #pragma unroll
-          for (int r = 0; r < 16; ++r) s[nb][r] = 0.f;
+    for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8 af = frag_rowmajor<D>(kt, kb, ks, lane);
+      for (int nb = 0; nb < NQB; ++nb) s[nb] = mfma32(kf[ks], qreg[nb][ks], s[nb]);
+    bf16x8 vT[MB][2];
 #pragma unroll
-          for (int nb = 0; nb < NQB; ++nb) s[nb] = mfma32(af, qreg[nb][ks], s[nb]);
-        }
-        const bool need_mask = (p.causal && jb + 31 > qw0 + p.q_start) || jb + 32 > p.Sk;
-        if (need_mask) {
+    for (int mb = 0; mb < MB; ++mb) {
+      vT[mb][0] = swz_frag_tr<D>(tr, mb, 2 * kb);
+      vT[mb][1] = swz_frag_tr<D>(tr, mb, 2 * kb + 1);
+    }
+    if (MASKED) {  // block touches the diagonal or the end of the keys
 #pragma unroll
-          for (int nb = 0; nb < NQB; ++nb) {
-            const int qlim = p.causal ? min(qw0 + 32 * nb + ln + p.q_start, p.Sk - 1) : p.Sk - 1;
-            // register r holds key jb + 4hh + c_r, c_r = 8(r/4) + r%4: masked iff c_r > qlim - jb - 4hh
-            const int t = qlim - jb - 4 * hh;
+      for (int nb = 0; nb < NQB; ++nb) {
+        // register r holds key jb + 4hh + c_r, c_r = 8(r/4) + r%4: masked iff c_r > qlim - jb - 4hh
+        const int t = qlim[nb] - jb - 4 * hh;
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-              if (8 * (r >> 2) + (r & 3) > t) s[nb][r] = -INFINITY;
-          }
-        }
-        if (!bounded) {
-          // general path: lazily maintained reference, raised only when a row exceeds it by 2^kLazyThresh
-#pragma unroll
-          for (int nb = 0; nb < NQB; ++nb) {
-            float mx = s[nb][0];
-#pragma unroll
-            for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[nb][r]);
-            mx = half_max(mx);
-            const bool need = mx > m_ref[nb] + kLazyThresh;
-            if (__builtin_amdgcn_ballot_w64(need) != 0) {
-              const float m_new = need ? mx : m_ref[nb];
-              const float corr = fast_exp2(m_ref[nb] - m_new);
-              m_ref[nb] = m_new;
-              l_run[nb] *= corr;
-#pragma unroll
-              for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[mb][nb][r] *= corr;
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[nb][r] -= m_ref[nb];
-          }
-        }
-        bf16x8 pb[2][NQB];
-#pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[nb][r] = fast_exp2(s[nb][r]);
-          pb[0][nb] = pack_c_half_sum(s[nb], 0, l_run[nb]);
-          pb[1][nb] = pack_c_half_sum(s[nb], 1, l_run[nb]);
-        }
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) {
-            const bf16x8 vf = frag_transposed<D>(vt, mb, 2 * kb + s2, lane);
-#pragma unroll
-            for (int nb = 0; nb < NQB; ++nb) oacc[mb][nb] = mfma32(vf, pb[s2][nb], oacc[mb][nb]);
-          }
+        for (int r = 0; r < 16; ++r)
+          if (8 * (r >> 2) + (r & 3) > t) s[nb][r] = -INFINITY;
       }
     }
-    if (more) {
-      uint16_t* nk = lds + ((jt + 1) & 1) * 2 * T::kElems;
-      stage_store<D, VR>(sr, nk, nk + T::kElems, p.eps, c1, c2);
+    if (!BOUNDED) {
+      // general path: lazily maintained reference, raised only when a row exceeds it by 2^kLazyThresh
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb) {
+        float mx = s[nb][0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[nb][r]);
+        mx = half_max(mx);
+        const bool need = mx > m_ref[nb] + kLazyThresh;
+        if (__builtin_amdgcn_ballot_w64(need) != 0) {
+          const float m_new = need ? mx : m_ref[nb];
+          const float corr = fast_exp2(m_ref[nb] - m_new);
+          m_ref[nb] = m_new;
+          l_run[nb] *= corr;
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[mb][nb][r] *= corr;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[nb][r] -= m_ref[nb];
+      }
     }
+    bf16x8 pb[2][NQB];
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[nb][r] = fast_exp2(s[nb][r]);
+      pb[0][nb] = pack_c_half_sum(s[nb], 0, l_run[nb]);
+      pb[1][nb] = pack_c_half_sum(s[nb], 1, l_run[nb]);
+    }
+    if (more) request_rowmajor(next_rm, next_kb);
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) oacc[mb][nb] = mfma32(vT[mb][s2], pb[s2][nb], oacc[mb][nb]);
+  };
+
+  // leading blocks of this wave that need no mask: every key of the block is visible to every query of the
+  // wave and lies inside the key range
+  int n_full = p.Sk / 32;
+  if (p.causal) n_full = min(n_full, (qw0 + p.q_start + 1) / 32);
+
+  // ---- pipeline.  All earlier vector loads are drained first: the tile loads that stay in flight across
+  // iterations must be the youngest vector-memory operations of the wave (waits are in-order).
+  // Protocol: at the top of iteration jt tiles jt and jt+1 have landed and tiles jt+2 .. jt+NS-2 are in
+  // flight; the stage of tile jt-1 is free (everyone passed the barrier that ended iteration jt-1), so tile
+  // jt+NS-1 is requested right away and has a whole iteration to land; the wait at the bottom leaves the
+  // youngest NS-3 tiles in flight, i.e. tile jt+2 is complete before the barrier.
+  auto run = [&](auto bounded_c) {
+    drain_vector_loads();
+#pragma unroll
+    for (int t = 0; t < NS - 1; ++t)
+      if (t < n_kt) issue_tile(t);
+    if (n_kt >= NS - 1) wait_vmcnt<(NS - 3) * kLoadsPerTile>(); else wait_vmcnt<0>();  // tiles 0 and 1 have landed
     __syncthreads();
-  }
+    if (n_act > 0) request_rowmajor(rm_lane, 0);
+    int stage = 0;
+    for (int jt = 0; jt < n_kt; ++jt) {
+      const int nstage = stage == NS - 1 ? 0 : stage + 1;
+      const bool issued = jt + NS - 1 < n_kt;
+      if (issued) issue_tile(jt + NS - 1);
+      const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
+      const uint32_t rm_next = rm_lane + nstage * kStageBytes;
+      const int blk = 2 * jt;
+      if (blk < n_act) {
+        if (blk < n_full) step(IC<0>{}, bounded_c, tr, 0, 32 * blk, blk + 1 < n_act, rm, 1);
+        else step(IC<1>{}, bounded_c, tr, 0, 32 * blk, blk + 1 < n_act, rm, 1);
+      }
+      if (blk + 1 < n_act) {
+        if (blk + 1 < n_full) step(IC<0>{}, bounded_c, tr, 1, 32 * blk + 32, blk + 2 < n_act, rm_next, 0);
+        else step(IC<1>{}, bounded_c, tr, 1, 32 * blk + 32, blk + 2 < n_act, rm_next, 0);
+      }
+      if (issued) wait_vmcnt<(NS - 3) * kLoadsPerTile>(); else wait_vmcnt<0>();
+      __syncthreads();
+      stage = nstage;
+    }
+  };
+  if (bounded) run(IC<1>{}); else run(IC<0>{});
 
   // ---- epilogue: normalise, gate, store y (bf16) and lse (fp32, natural log)
 #pragma unroll
@@ -225,40 +271,27 @@ __global__ __launch_bounds__(kThreadsM, SEGPT_FWD_OCC) void fwd_bf16_kernel(KArg
     uint16_t* op = live ? row_ptr_mut<uint16_t>(p.o, b, h, row) : nullptr;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
+      float val[16];
 #pragma unroll
-      for (int cc = 0; cc < 2; ++cc) {
-        // registers 8cc..8cc+3 hold d = 32mb+16cc+4hh+{0..3}; 8cc+4..8cc+7 hold d = 32mb+16cc+8+4hh+{0..3}
-        const f32x16& o = oacc[mb][nb];
-        const uint32_t x0 = pack_bf16x2(o[8 * cc + 0] * f, o[8 * cc + 1] * f);
-        const uint32_t x1 = pack_bf16x2(o[8 * cc + 2] * f, o[8 * cc + 3] * f);
-        const uint32_t y0 = pack_bf16x2(o[8 * cc + 4] * f, o[8 * cc + 5] * f);
-        const uint32_t y1 = pack_bf16x2(o[8 * cc + 6] * f, o[8 * cc + 7] * f);
-        // lanes < 32 end up with d = 32mb+16cc+0..7, lanes >= 32 with d = 32mb+16cc+8..15
-        auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
-        auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-        const u32x4 w = {s0[0], s1[0], s0[1], s1[1]};
-        if (live) *reinterpret_cast<u32x4*>(op + 32 * mb + 16 * cc + 8 * hh) = w;
-      }
+      for (int r = 0; r < 16; ++r) val[r] = oacc[mb][nb][r] * f;
+      store_ct_block(op, mb, hh, live, val);
     }
   }
 }
 
-template <int D, int NQB>
+template <int D>
 int launch_fwd_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
-  constexpr int BQ = FwdCfg<D, NQB>::kBQ;
-  const int n_qt = (p.Sq + BQ - 1) / BQ;
-  dim3 grid((unsigned)(n_qt * p.H * p.B)), block(kThreadsM);
-  if (p.v_first.ptr) hipLaunchKernelGGL((fwd_bf16_kernel<D, NQB, true>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((fwd_bf16_kernel<D, NQB, false>), grid, block, 0, st, a);
+  const int n_qt = (p.Sq + FwdShape<D>::kBQ - 1) / FwdShape<D>::kBQ;
+  hipLaunchKernelGGL((fwd_bf16_kernel<D>), dim3((unsigned)(n_qt * p.H * p.B)), dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 
 }  // namespace
 
 int launch_fwd_bf16(const KArgs& a, hipStream_t st) {
-  if (a.p.D == 64) return launch_fwd_t<64, SEGPT_FWD_NQB>(a, st);
-  if (a.p.D == 128) return launch_fwd_t<128, 1>(a, st);
+  if (a.p.D == 64) return launch_fwd_t<64>(a, st);
+  if (a.p.D == 128) return launch_fwd_t<128>(a, st);
   return (int)hipErrorInvalidValue;
 }
 

@@ -25,15 +25,6 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kBK = 64;        // streamed rows per LDS tile
 constexpr int kThreadsM = 256; // 4 waves
 
-template <int D>
-struct Tile {
-  static constexpr int kRS = D + 8;                 // LDS row stride in bf16 elements (16 B pad)
-  static constexpr int kElems = kBK * kRS;          // elements of one staged tile
-  static constexpr int kTPR = D / 8;                // threads per row when staging (16 B each)
-  static constexpr int kRowsPerPass = kThreadsM / kTPR;
-  static constexpr int kPasses = kBK / kRowsPerPass;  // 16-byte loads per thread per tile
-};
-
 __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
@@ -63,23 +54,6 @@ __device__ __forceinline__ void drain_vector_loads() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-// x + (x of another lane) through a DPP lane pattern (no LDS traffic, fuses into v_add_f32_dpp)
-template <int CTRL>
-__device__ __forceinline__ float dpp_add(float x) {
-  return x + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
-}
-
-// sum over the kTPR (8 or 16) adjacent lanes that stage one row; every lane of the group gets the total
-template <int TPR>
-__device__ __forceinline__ float row_group_sum(float x) {
-  static_assert(TPR == 8 || TPR == 16, "row groups are 8 or 16 lanes");
-  x = dpp_add<0xB1>(x);   // quad_perm [1,0,3,2]
-  x = dpp_add<0x4E>(x);   // quad_perm [2,3,0,1]
-  x = dpp_add<0x141>(x);  // row_half_mirror: the other quad of the 8-lane half row
-  if (TPR == 16) x = dpp_add<0x140>(x);  // row_mirror: the other half of the 16-lane row
-  return x;
-}
-
 // acc + lo + hi of one packed bf16 pair (v_dot2c_f32_bf16 with a (1,1) operand): sums the ROUNDED values,
 // i.e. exactly what the MFMA consuming the packed operand sees.
 __device__ __forceinline__ float add_bf16_pair(uint32_t w, float acc) {
@@ -103,70 +77,6 @@ __device__ __forceinline__ u32x4 scale8(u32x4 v, float f) {
   for (int i = 0; i < 4; ++i) r[i] = pack_bf16x2(bf16lo(v[i]) * f, bf16hi(v[i]) * f);
   return r;
 }
-__device__ __forceinline__ u32x4 mix8(u32x4 a, u32x4 b, float ca, float cb) {
-  u32x4 r;
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-    r[i] = pack_bf16x2(ca * bf16lo(a[i]) + cb * bf16lo(b[i]), ca * bf16hi(a[i]) + cb * bf16hi(b[i]));
-  return r;
-}
-
-// A/B fragment of a row-major LDS tile for the 32-row block `rb`, contraction step `ks` (16 columns):
-// lane reads 16 contiguous bytes at row 32*rb + l%32, column 16*ks + 8*(l/32).
-template <int D>
-__device__ __forceinline__ bf16x8 frag_rowmajor(const uint16_t* tile, int rb, int ks, int lane) {
-  const uint16_t* p = tile + (32 * rb + (lane & 31)) * Tile<D>::kRS + 16 * ks + 8 * (lane >> 5);
-  return as_bf16x8(*reinterpret_cast<const u32x4*>(p));
-}
-
-// Transposed fragment of a row-major LDS tile [row][col]: the lane's MFMA row is a COLUMN of the tile
-// (col = 32*cb + l%32) and its 8 contraction entries are tile rows in CPERM order
-//   16*s + {4hh..4hh+3, 8+4hh..8+4hh+3}.
-// ds_read_b64_tr_b16 semantics (per 16-lane group, source lane r gives the address of 4 elements):
-//   result[lane i][e] = LDS[addr(4e + i/4) + i%4]
-// so source lane r points at row base + r/4, column cbase + 4*(r%4) and lane i receives column cbase + i,
-// rows base..base+3.
-template <int D>
-__device__ __forceinline__ bf16x8 frag_transposed(const uint16_t* tile, int cb, int s, int lane) {
-  const int r = lane & 15;
-  const int hh = lane >> 5;
-  const int col = 32 * cb + 16 * ((lane >> 4) & 1) + 4 * (r & 3);
-  const int row = 16 * s + 4 * hh + (r >> 2);
-  const uint16_t* p = tile + row * Tile<D>::kRS + col;
-  typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
-  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
-  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 8 * Tile<D>::kRS));
-  typedef short s16x8 __attribute__((ext_vector_type(8)));
-  s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  return __builtin_bit_cast(bf16x8, v);
-}
-
-// ---- the same two fragment readers with every term but one per-lane base folded into the instruction's
-// immediate offset: `base` = LDS byte address of the tile + lane_off_rm / lane_off_tr, block indices constant.
-template <int D>
-__device__ __forceinline__ int lane_off_rm(int lane) {
-  return ((lane & 31) * Tile<D>::kRS + 8 * (lane >> 5)) * 2;
-}
-template <int D>
-__device__ __forceinline__ int lane_off_tr(int lane) {
-  const int r = lane & 15;
-  return ((4 * (lane >> 5) + (r >> 2)) * Tile<D>::kRS + 16 * ((lane >> 4) & 1) + 4 * (r & 3)) * 2;
-}
-template <int D>
-__device__ __forceinline__ bf16x8 frag_rm_at(const char* base, int rb, int ks) {
-  return as_bf16x8(*reinterpret_cast<const u32x4*>(base + (32 * rb * Tile<D>::kRS + 16 * ks) * 2));
-}
-template <int D>
-__device__ __forceinline__ bf16x8 frag_tr_at(const char* base, int cb, int s) {
-  const char* p = base + (16 * s * Tile<D>::kRS + 32 * cb) * 2;
-  typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
-  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
-  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 8 * Tile<D>::kRS * 2));
-  typedef short s16x8 __attribute__((ext_vector_type(8)));
-  s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  return __builtin_bit_cast(bf16x8, v);
-}
-
 // ---------------------------------------------------------------------------------------------------
 // Swizzled, unpadded LDS tiles filled by direct global->LDS loads (global_load_lds_dwordx4: every lane
 // names its own 16 global bytes, the wave's 64 x 16 B land contiguously at a wave-uniform LDS address).
@@ -245,6 +155,12 @@ __device__ __forceinline__ int swz_off_rm(int lane) {
   const int ln = lane & 31, hh = lane >> 5;
   return ln * Swz<D>::kRB + ((hh ^ Swz<D>::f(ln)) << 4);
 }
+// Transposed fragment of a row-major tile [row][col]: the lane's MFMA row is a COLUMN of the tile
+// (col = 32*cb + l%32) and its 8 contraction entries are tile rows in CPERM order 16*s + {4hh..4hh+3, 8+4hh..8+4hh+3}.
+// ds_read_b64_tr_b16 semantics (per 16-lane group, source lane r gives the address of 4 elements):
+//   result[lane i][e] = LDS[addr(4e + i/4) + i%4]
+// so source lane r points at row base + r/4, column cbase + 4*(r%4) and lane i receives column cbase + i,
+// rows base..base+3.
 // Per-lane byte offset of the transposed fragment of column block 0, row step 0 (first of its two
 // 8-byte reads; the second is 8 rows further, which also flips kHiXor in the swizzle term): column block
 // cb is this offset XOR (cb << 6), row step s adds 16*s*kRB.
@@ -294,44 +210,61 @@ __device__ __forceinline__ bf16x8 pack_c_half_sum(const f32x16& c, int s, float&
   return as_bf16x8(w);
 }
 
-// ---- K/V tile staging: global -> registers (16 B per thread per pass) -> normalise / mix -> LDS (row-major)
-template <int D>
-struct StageRegs {
-  u32x4 k[Tile<D>::kPasses], v[Tile<D>::kPasses], vf[Tile<D>::kPasses];
-};
+// ---- helpers shared by the ring kernels (forward, dQ, dK/dV)
+__device__ __forceinline__ float gprod_at(const segpt_attn_params& p, int d) {
+  float g = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
+  if (p.gk_numel == 1) g *= p.g_k[0];
+  else if (p.gk_numel > 1) g *= p.g_k[d];
+  return g;
+}
 
-template <int D, bool VR>
-__device__ __forceinline__ void stage_load(const segpt_attn_params& p, int b, int g, int j0, StageRegs<D>& r) {
-  using T = Tile<D>;
-  const int tid = threadIdx.x;
-  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
+// store a C tile column block: lane = row of the output tensor, registers = 32 consecutive columns
+// starting at 32*mb, values already scaled.  Lanes l and l^32 exchange halves so that each lane
+// writes 16 contiguous bytes.
+__device__ __forceinline__ void store_ct_block(uint16_t* rowp, int mb, int hh, bool live, const float (&val)[16]) {
 #pragma unroll
-  for (int ps = 0; ps < T::kPasses; ++ps) {
-    const int j = j0 + r0 + ps * T::kRowsPerPass;
-    if (j < p.Sk) {
-      r.k[ps] = *reinterpret_cast<const u32x4*>(row_ptr<uint16_t>(p.k, b, g, j) + chunk * 8);
-      r.v[ps] = *reinterpret_cast<const u32x4*>(row_ptr<uint16_t>(p.v, b, g, j) + chunk * 8);
-      if (VR) r.vf[ps] = *reinterpret_cast<const u32x4*>(row_ptr<uint16_t>(p.v_first, b, g, j) + chunk * 8);
-    } else {
-      r.k[ps] = u32x4{0, 0, 0, 0};
-      r.v[ps] = u32x4{0, 0, 0, 0};
-      if (VR) r.vf[ps] = u32x4{0, 0, 0, 0};
-    }
+  for (int cc = 0; cc < 2; ++cc) {
+    const uint32_t x0 = pack_bf16x2(val[8 * cc + 0], val[8 * cc + 1]);
+    const uint32_t x1 = pack_bf16x2(val[8 * cc + 2], val[8 * cc + 3]);
+    const uint32_t y0 = pack_bf16x2(val[8 * cc + 4], val[8 * cc + 5]);
+    const uint32_t y1 = pack_bf16x2(val[8 * cc + 6], val[8 * cc + 7]);
+    auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+    auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+    const u32x4 w = {s0[0], s1[0], s0[1], s1[1]};
+    if (live) *reinterpret_cast<u32x4*>(rowp + 32 * mb + 16 * cc + 8 * hh) = w;
   }
 }
 
-template <int D, bool VR>
-__device__ __forceinline__ void stage_store(const StageRegs<D>& r, uint16_t* kt, uint16_t* vt, float eps, float c1, float c2) {
-  using T = Tile<D>;
-  const int tid = threadIdx.x;
-  const int chunk = tid % T::kTPR, r0 = tid / T::kTPR;
+// raw bf16 values of a tensor row at the 16 columns a lane's C registers of block mb map to
+__device__ __forceinline__ void load_ct_block(const uint16_t* rowp, int mb, int hh, float (&out)[16]) {
 #pragma unroll
-  for (int ps = 0; ps < T::kPasses; ++ps) {
-    const int row = r0 + ps * T::kRowsPerPass;
-    const float ss = row_group_sum<T::kTPR>(sumsq8(r.k[ps]));
-    const float beta = fast_rsq(ss * (1.0f / D) + eps);
-    *reinterpret_cast<u32x4*>(kt + row * T::kRS + chunk * 8) = scale8(r.k[ps], beta);
-    *reinterpret_cast<u32x4*>(vt + row * T::kRS + chunk * 8) = VR ? mix8(r.v[ps], r.vf[ps], c1, c2) : r.v[ps];
+  for (int c = 0; c < 4; ++c) {
+    const u32x2 w = *reinterpret_cast<const u32x2*>(rowp + 32 * mb + 8 * c + 4 * hh);
+    out[4 * c + 0] = bf16lo(w[0]); out[4 * c + 1] = bf16hi(w[0]);
+    out[4 * c + 2] = bf16lo(w[1]); out[4 * c + 3] = bf16hi(w[1]);
+  }
+}
+
+__device__ __forceinline__ f32x16 splat16(float x) {
+  f32x16 v;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) v[r] = x;
+  return v;
+}
+
+// Issue the direct global->LDS loads of two [64, D] bf16 tiles (rows row0..row0+63 of two row-major
+// tensors; rows past nrows re-read the last valid row, callers mask them) into one stage.
+//   src_a/src_b: wave-uniform pointers to row `row0` of each tensor; step_*: bytes between rows
+//   dst: LDS byte address of the stage + wave*1024 (wave-uniform); lane_row / lane_col: from swz_src()
+template <int D>
+__device__ __forceinline__ void issue_tile_pair(const char* src_a, uint32_t step_a, const char* src_b, uint32_t step_b,
+                                                int rows_left, uint32_t dst, int lane_row, int lane_col) {
+  using Z = Swz<D>;
+#pragma unroll
+  for (int ps = 0; ps < Z::kPasses; ++ps) {
+    const int row = min(lane_row + ps * 4 * Z::kRowsPerInst, rows_left - 1);
+    gload_lds16(src_a + (uint32_t)row * step_a + lane_col, dst + ps * 4096);
+    gload_lds16(src_b + (uint32_t)row * step_b + lane_col, dst + Z::kTileBytes + ps * 4096);
   }
 }
 

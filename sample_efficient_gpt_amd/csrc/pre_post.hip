@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256) void bwd_pre_kernel(KArgs a) {
 
 // bf16 path: Khat = b_j k_j and (with a value residual) V' = c1 v + c2 v_first, one row per 8/16 lanes
 template <int D>
-__global__ __launch_bounds__(256) void bwd_prep_kv_kernel(KArgs a) {
+__global__ __launch_bounds__(256) void kv_prep_kernel(KArgs a) {
   const segpt_attn_params& p = a.p;
   constexpr int TPR = D / 8;
   constexpr int RPB = 256 / TPR;
@@ -217,14 +217,19 @@ int launch_pre_t(const KArgs& a, hipStream_t st) {
 }  // namespace
 
 int launch_bwd_pre(const KArgs& a, hipStream_t st) {
-  if (a.p.dtype == SEGPT_DTYPE_FP32) return launch_pre_t<float>(a, st);
-  // bf16: the per-query-row quantities (delta, Qhat, gate terms) come from the dQ kernel's prologue
+  if (a.p.dtype != SEGPT_DTYPE_FP32) return (int)hipErrorInvalidValue;
+  return launch_pre_t<float>(a, st);
+}
+
+// bf16: the per-key-row pre-pass shared by forward and backward (the per-query-row quantities of the backward,
+// delta / Qhat / gate terms, come from the dQ kernel's prologue)
+int launch_kv_prep(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
   const int64_t nrows = (int64_t)p.B * p.Hkv * p.Sk;
   const int rpb = 256 / (p.D / 8);
   dim3 grid((unsigned)((nrows + rpb - 1) / rpb)), block(256);
-  if (p.D == 64) hipLaunchKernelGGL(bwd_prep_kv_kernel<64>, grid, block, 0, st, a);
-  else hipLaunchKernelGGL(bwd_prep_kv_kernel<128>, grid, block, 0, st, a);
+  if (p.D == 64) hipLaunchKernelGGL(kv_prep_kernel<64>, grid, block, 0, st, a);
+  else hipLaunchKernelGGL(kv_prep_kernel<128>, grid, block, 0, st, a);
   return (int)hipGetLastError();
 }
 

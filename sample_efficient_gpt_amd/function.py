@@ -71,21 +71,25 @@ def _check_inputs(q, k, v, g_q, g_k, v_first, vr_coef, gate):
 
 
 def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y):
-    """Launch the forward on canonical 4-D views; returns lse [B,H,Sq] fp32.  `y` is written."""
+    """Launch the forward on canonical 4-D views; returns (lse [B,H,Sq] fp32, kv workspace).  `y` is written.
+    The kv workspace holds the normalised keys (and mixed values) the backward can reuse."""
     lib = _lib.load()
     B, H, Sq, _ = q.shape
     lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
     p = _lib.new_params()
     _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start)
+    kv_ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_KV, q.device)
+    p.kv_workspace, p.kv_workspace_bytes = kv_ws.data_ptr(), kv_ws.numel()
     rc = lib.segpt_attn_fwd(p, torch.cuda.current_stream(q.device).cuda_stream)
     if rc != 0:
         raise _lib.SegptError(rc, "segpt_attn_fwd")
-    return lse
+    return lse, kv_ws
 
 
 def _backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y, lse, dy,
-              dq, dk, dv, dv_first, dgate):
-    """Launch the backward; dq/dk/dv(/dv_first/dgate) are written; returns (dg_q, dg_k, dvr_coef) fp32."""
+              dq, dk, dv, dv_first, dgate, kv_ws=None):
+    """Launch the backward; dq/dk/dv(/dv_first/dgate) are written; returns (dg_q, dg_k, dvr_coef) fp32.
+    `kv_ws`: the forward's kv workspace (skips the key/value pre-pass); None allocates a fresh one."""
     lib = _lib.load()
     dev = q.device
     dg_q = torch.empty_like(g_q)
@@ -97,9 +101,13 @@ def _backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_sca
     p.dv_first = _lib.t4(dv_first)
     p.dgate = _lib.t3(dgate)
     p.dg_q, p.dg_k, p.dvr_coef = _lib.ptr(dg_q), _lib.ptr(dg_k), _lib.ptr(dcoef)
-    nbytes = lib.segpt_attn_workspace_bytes(p, 1)
-    ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=dev)
+    ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_BWD, dev)
     p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    if kv_ws is None:
+        kv_ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_KV, dev)
+    else:
+        p.flags = _lib.SEGPT_FLAG_KV_PREPARED
+    p.kv_workspace, p.kv_workspace_bytes = kv_ws.data_ptr(), kv_ws.numel()
     rc = lib.segpt_attn_bwd(p, torch.cuda.current_stream(dev).cuda_stream)
     if rc != 0:
         raise _lib.SegptError(rc, "segpt_attn_bwd")
@@ -125,15 +133,16 @@ class _CoreFunc(torch.autograd.Function):
         y = torch.empty_like(q)
         if y.stride(-1) != 1:
             y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-        lse = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y)
-        ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse)
+        lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y)
+        # the normalised keys (bf16 path) are kept for the backward: 1/rep of q's size
+        ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse, kv_ws)
         ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start)
         ctx.mark_non_differentiable(lse)
         return y, lse
 
     @staticmethod
     def backward(ctx, dy, _dlse):
-        q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse = ctx.saved_tensors
+        q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse, kv_ws = ctx.saved_tensors
         gate_scale, eps, sm_scale, causal, q_start = ctx.cfg
         gq32, gk32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device)
         coef32 = None if vr_coef is None else vr_coef.detach().to(device=q.device, dtype=torch.float32).reshape(-1).contiguous()
@@ -144,7 +153,7 @@ class _CoreFunc(torch.autograd.Function):
         dv_first = None if v_first is None else torch.empty_like(v_first)
         dgate = None if gate is None else torch.empty_like(gate)
         dg_q, dg_k, dcoef = _backward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal,
-                                      q_start, y, lse, dy, dq, dk, dv, dv_first, dgate)
+                                      q_start, y, lse, dy, dq, dk, dv, dv_first, dgate, kv_ws)
         dg_q = dg_q.reshape(g_q.shape).to(g_q.dtype)
         if g_k is not None:
             dg_k = dg_k.reshape(g_k.shape).to(g_k.dtype)
@@ -215,15 +224,15 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
         if sm_scale is None:
             sm_scale = 1.0 / math.sqrt(Q.shape[-1])
         O = torch.empty_like(Q)
-        lse = _forward(q4, k4, v4, gq32, gk32, vf4, coef32, gate_logits, gate_scale, eps, sm_scale, is_causal, q_start,
-                       _canon(O, H))
-        ctx.save_for_backward(lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate_logits)
+        lse, kv_ws = _forward(q4, k4, v4, gq32, gk32, vf4, coef32, gate_logits, gate_scale, eps, sm_scale, is_causal,
+                              q_start, _canon(O, H))
+        ctx.save_for_backward(lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate_logits, kv_ws)
         ctx.cfg = (H, Hkv, gate_scale, eps, sm_scale, bool(is_causal), int(q_start))
         return O
 
     @staticmethod
     def backward(ctx, grad_output):
-        lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate = ctx.saved_tensors
+        lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate, kv_ws = ctx.saved_tensors
         H, Hkv, gate_scale, eps, sm_scale, causal, q_start = ctx.cfg
         grad_output = grad_output.contiguous()
         if grad_output.dtype != Q.dtype:
@@ -239,7 +248,7 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
             _canon(Q, H), _canon(K, Hkv), _canon(V, Hkv), gq32, gk32,
             None if v_first is None else _canon(v_first, Hkv), coef32, gate, gate_scale, eps, sm_scale, causal, q_start,
             _canon(O, H), lse, _canon(grad_output, H), _canon(dQ, H), _canon(dK, Hkv), _canon(dV, Hkv),
-            None if dVf is None else _canon(dVf, Hkv), dgate)
+            None if dVf is None else _canon(dVf, Hkv), dgate, kv_ws)
         dgain = dg_q.reshape(gain.shape).to(gain.dtype)
         dk_gain = None if k_gain is None else dg_k.reshape(k_gain.shape).to(k_gain.dtype)
         dcoef = None if vr_coef is None else dcoef.reshape(vr_coef.shape).to(vr_coef.dtype)

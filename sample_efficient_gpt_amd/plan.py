@@ -31,6 +31,8 @@ class AttnPlan:
         p = _lib.new_params()
         _fill_common(p, q, k, v, self.y, self.lse, self.g_q, self.g_k, self.v_first, self.coef, self.gate, gate_scale,
                      eps, sm_scale, causal, q_start)
+        self.kv_ws = _lib.alloc_workspace(self.lib, p, _lib.SEGPT_WS_KV, dev)
+        p.kv_workspace, p.kv_workspace_bytes = self.kv_ws.data_ptr(), self.kv_ws.numel()
         self.p = p
         self.has_bwd = backward
         if backward:
@@ -44,20 +46,29 @@ class AttnPlan:
             p.d_o, p.dq, p.dk, p.dv = _lib.t4(self.d_o), _lib.t4(self.dq), _lib.t4(self.dk), _lib.t4(self.dv)
             p.dv_first, p.dgate = _lib.t4(self.dv_first), _lib.t3(self.dgate)
             p.dg_q, p.dg_k, p.dvr_coef = _lib.ptr(self.dg_q), _lib.ptr(self.dg_k), _lib.ptr(self.dcoef)
-            nbytes = max(int(self.lib.segpt_attn_workspace_bytes(p, 1)), 256)
-            self.ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-            p.workspace, p.workspace_bytes = self.ws.data_ptr(), nbytes
+            self.ws = _lib.alloc_workspace(self.lib, p, _lib.SEGPT_WS_BWD, dev)
+            p.workspace, p.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
         self.stream = torch.cuda.current_stream(dev).cuda_stream
 
     def _chk(self, rc, what):
         if rc != 0:
             raise _lib.SegptError(rc, what)
 
-    def forward(self):
+    def forward(self, flags: int = 0):
+        """Key/value pre-pass + attention kernel; leaves the normalised keys in the plan's kv workspace."""
+        self.p.flags = flags
         self._chk(self.lib.segpt_attn_fwd(self.p, self.stream), "segpt_attn_fwd")
 
-    def backward(self):
+    def forward_stage(self, stage: int):
+        self.p.flags = 0
+        self._chk(self.lib.segpt_attn_fwd_stage(self.p, stage, self.stream), "segpt_attn_fwd_stage")
+
+    def backward(self, kv_prepared: bool = False):
+        """`kv_prepared`: forward() ran on this plan since k / v last changed, so the backward reuses its
+        normalised keys instead of running the pre-pass again."""
+        self.p.flags = _lib.SEGPT_FLAG_KV_PREPARED if kv_prepared else 0
         self._chk(self.lib.segpt_attn_bwd(self.p, self.stream), "segpt_attn_bwd")
 
-    def backward_stage(self, stage: int):
+    def backward_stage(self, stage: int, kv_prepared: bool = False):
+        self.p.flags = _lib.SEGPT_FLAG_KV_PREPARED if kv_prepared else 0
         self._chk(self.lib.segpt_attn_bwd_stage(self.p, stage, self.stream), "segpt_attn_bwd_stage")

@@ -60,6 +60,7 @@ def _valid_params(dtype=_lib.SEGPT_DTYPE_BF16, D=64):
     for name in ("k", "v", "dk", "dv"):
         setattr(p, name, _lib.Tensor4(fake, 2 * 128 * D, 128 * D, D))
     p.lse = p.g_q = p.dg_q = fake
+    p.kv_workspace, p.kv_workspace_bytes = 0x40000, 1 << 30
     return p
 
 
@@ -93,6 +94,14 @@ def test_argument_errors_are_reported_before_any_launch(lib):
     assert lib.segpt_attn_fwd(p, None) == -1
     p = _valid_params(); p.v_first = _lib.Tensor4(0x10000, 2 * 128 * 64, 128 * 64, 64)  # v_first without vr_coef
     assert lib.segpt_attn_fwd(p, None) == -8
+    p = _valid_params(); p.kv_workspace = None
+    assert lib.segpt_attn_fwd(p, None) == -7  # bf16 needs the key/value workspace
+    p = _valid_params(); p.kv_workspace_bytes = lib.segpt_attn_workspace_bytes(p, _lib.SEGPT_WS_KV) - 1
+    assert lib.segpt_attn_fwd(p, None) == -7
+    p = _valid_params(); p.kv_workspace = 0x40010
+    assert lib.segpt_attn_fwd(p, None) == -10
+    assert lib.segpt_attn_fwd_stage(_valid_params(), 2, None) == -11
+    assert lib.segpt_attn_bwd_stage(_valid_params(), 4, None) == -11
     # backward-only checks
     p = _valid_params()
     assert lib.segpt_attn_bwd(p, None) == -7  # no workspace
@@ -108,8 +117,14 @@ def test_argument_errors_are_reported_before_any_launch(lib):
 
 def test_workspace_bytes(lib):
     p = _valid_params()
-    assert lib.segpt_attn_workspace_bytes(p, 0) == 0
-    base = lib.segpt_attn_workspace_bytes(p, 1)
+    kv = lib.segpt_attn_workspace_bytes(p, _lib.SEGPT_WS_KV)
+    assert kv >= 2 * 2 * 128 * 64 * 2 and kv % 256 == 0  # normalised keys [B,Hkv,Sk,D] bf16
+    p.v_first = _lib.Tensor4(0x10000, 2 * 128 * 64, 128 * 64, 64)
+    assert lib.segpt_attn_workspace_bytes(p, _lib.SEGPT_WS_KV) >= 2 * kv  # + mixed values
+    assert lib.segpt_attn_workspace_bytes(_valid_params(dtype=_lib.SEGPT_DTYPE_FP32), _lib.SEGPT_WS_KV) == 0
+    assert lib.segpt_attn_workspace_bytes(p, 2) == 0
+    p = _valid_params()
+    base = lib.segpt_attn_workspace_bytes(p, _lib.SEGPT_WS_BWD)
     rows = 2 * 6 * 128
     assert base >= rows * 4 and base % 256 == 0
     p.gate = _lib.Tensor3(0x10000, 128 * 6, 6, 1)

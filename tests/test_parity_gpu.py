@@ -147,6 +147,77 @@ def test_cfg5_wide_head_full_size(gpu_device):
     _slice_check(gpu_device, CONFIGS[5], [(0, 0), (3, 3)])
 
 
+def test_running_maximum_path(gpu_device):
+    """The forward has two softmax paths: raw exp2 when the QK-norm bound on the logits allows it, and a lazily
+    raised running maximum otherwise.  (a) Forced onto the second path, ordinary inputs must meet the same
+    tolerance against the oracle and agree with the first path; (b) gains large enough to leave the bound
+    (sm_scale*log2e*D*max|g|*1.02 ~ 68 > 64) select it by themselves."""
+    from sample_efficient_gpt_amd import _lib
+    from sample_efficient_gpt_amd.plan import AttnPlan
+
+    x = gen(2, 4, 2, 320, 320, 64, BF16, seed=11)
+    ref = run_oracle(x, backward=False)
+    plan = AttnPlan({n: (t.to(gpu_device) if t is not None else None) for n, t in x.items()}, backward=False)
+    print("forced running-maximum path", flush=True)
+    plan.forward()
+    fast = {"y": plan.y.cpu(), "lse": plan.lse.cpu()}
+    plan.forward(flags=_lib.SEGPT_FLAG_RUNNING_MAX)
+    slow = {"y": plan.y.cpu(), "lse": plan.lse.cpu()}
+    compare(fast, ref, BF16)
+    compare(slow, ref, BF16)
+    assert torch.allclose(fast["y"].float(), slow["y"].float(), atol=4e-3, rtol=8e-3)  # one bf16 ulp of each other
+    # the row sum adds bf16-rounded probabilities, which round differently under a shifted reference point
+    assert torch.allclose(fast["lse"], slow["lse"], atol=4e-3, rtol=0)
+
+    x["g_q"] = x["g_q"] * 2.4
+    x["g_k"] = x["g_k"] * 2.4
+    assert float((x["g_q"] * x["g_k"]).abs().max()) * 0.125 * 1.4427 * 64 * 1.02 > 64.0
+    print("large-gain case", flush=True)
+    got = run_gpu(x, gpu_device, backward=False)
+    ref = run_oracle(x, backward=False)
+    # the bf16 rounding of Qhat and Khat perturbs a logit in proportion to the gain product (5.8x the ordinary
+    # case here), and P = exp(logit) inherits it: the absolute part of the tolerance is scaled accordingly
+    err = (got["y"].double() - ref["y"]).abs()
+    assert bool((err <= 5.8 * 2e-2 + 1e-2 * ref["y"].abs()).all()), float(err.max())
+    assert torch.allclose(got["lse"].double(), ref["lse"], atol=5.8 * 2e-2, rtol=1e-2)
+
+
+def test_plan_reuses_forward_kv_workspace_and_stages_match(gpu_device):
+    """C-ABI plan: backward with SEGPT_FLAG_KV_PREPARED (forward's normalised keys) == backward that runs its
+    own pre-pass == the stage-by-stage entry points, bit for bit; a forward without a kv workspace is refused."""
+    from sample_efficient_gpt_amd import _lib
+    from sample_efficient_gpt_amd.plan import AttnPlan
+
+    x = gen(2, 6, 2, 300, 300, 64, BF16, extras=True, seed=5)
+    xd = {n: (t.to(gpu_device) if t is not None else None) for n, t in x.items()}
+    plan = AttnPlan(xd, gate_scale=2.0)
+    outs = ("y", "lse", "dq", "dk", "dv", "dv_first", "dgate", "dg_q", "dg_k", "dcoef")
+    snap = lambda: {n: getattr(plan, n).clone() for n in outs}
+    plan.forward(); plan.backward(kv_prepared=True)
+    a = snap()
+    plan.kv_ws.zero_()  # a backward without the flag must rebuild the workspace itself
+    plan.backward(kv_prepared=False)
+    b = snap()
+    plan.kv_ws.zero_()
+    for n in outs:
+        getattr(plan, n).zero_()
+    for st in range(len(_lib.FWD_STAGES)):
+        plan.forward_stage(st)
+    for st in range(len(_lib.BWD_STAGES)):
+        plan.backward_stage(st)
+    c = snap()
+    torch.cuda.synchronize()
+    for n in outs:
+        assert torch.equal(a[n], b[n]), n
+        assert torch.equal(a[n], c[n]), n
+    ref = run_oracle(x, gate_scale=2.0)
+    compare({"y": a["y"].cpu(), "lse": a["lse"].cpu(), "dq": a["dq"].cpu(), "dk": a["dk"].cpu(), "dv": a["dv"].cpu()},
+            ref, BF16, names=["y", "lse", "dq", "dk", "dv"])
+    plan.p.kv_workspace = None
+    with pytest.raises(_lib.SegptError):
+        plan.forward()
+
+
 def test_backward_is_deterministic(gpu_device):
     x = gen(2, 6, 2, 512, 512, 64, BF16, extras=True, seed=4)
     a = run_gpu(x, gpu_device)
