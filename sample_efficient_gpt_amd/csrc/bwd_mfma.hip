@@ -54,7 +54,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   __shared__ __attribute__((aligned(16))) float red4[4 * D];  // per-wave column sums of the dg partial
   static_assert(kStages * kStageBytes >= 128 * (D + 1) * 4, "LDS reuse for the dg partial");
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: everything derived from it stays scalar
   const int ln = lane & 31, hh = lane >> 5;
   const int rep = p.H / p.Hkv;
   const int n_qt = (p.Sq + BQ - 1) / BQ;
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
 
   const uint32_t lds0 = lds_addr_of(lds);
   const int2 src = swz_src<D>(lane, wave);
-  const uint32_t wave_dst = lds0 + __builtin_amdgcn_readfirstlane(wave) * 1024;
+  const uint32_t wave_dst = lds0 + wave * 1024;
   auto issue_tile = [&](int jt) {  // tile jt -> stage jt % kStages
     issue_tile_pair<D>(kbase + (int64_t)jt * kBK * kstep, kstep, vbase + (int64_t)jt * kBK * vstep, vstep,
                        p.Sk - jt * kBK, wave_dst + (jt % kStages) * kStageBytes, src.x, src.y);
@@ -280,7 +281,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   __shared__ __attribute__((aligned(256))) float ldl[kStages * 128];  // per stage: [0,64) -lse2, [64,128) -delta
   __shared__ float red[8];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: everything derived from it stays scalar
   const int ln = lane & 31, hh = lane >> 5;
   const int rep = p.H / p.Hkv;
   const int n_kvt = (p.Sk + BKV - 1) / BKV;
@@ -304,9 +306,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   // of waves 0/1) so that one immediate vmcnt fits all.
   const uint32_t lds0 = lds_addr_of(lds), ldl0 = lds_addr_of(ldl);
   const int2 src = swz_src<D>(lane, wave);
-  const int uwave = __builtin_amdgcn_readfirstlane(wave);
   const bool do_contig = a.do_eff != nullptr;
-  const float* const stat_arr = (uwave & 1) ? a.delta : a.nlse2;
+  const float* const stat_arr = (wave & 1) ? a.delta : a.nlse2;
   auto issue_tile = [&](int it) {  // streamed tile it -> stage it % kStages
     const int hq = it / n_vis;
     const int i0 = (qt_start + it - hq * n_vis) * kBK;
@@ -317,8 +318,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
                                  : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, i0));
     const uint32_t dstep = do_contig ? (uint32_t)D * 2 : (uint32_t)p.d_o.stride_s * 2;
     const int stage = it % kStages;
-    issue_tile_pair<D>(qsrc, D * 2, dsrc, dstep, p.Sq - i0, lds0 + stage * kStageBytes + uwave * 1024, src.x, src.y);
-    gload_lds4(stat_arr + base + min(i0 + lane, p.Sq - 1), ldl0 + (stage * 128 + (uwave & 1) * 64) * 4);
+    issue_tile_pair<D>(qsrc, D * 2, dsrc, dstep, p.Sq - i0, lds0 + stage * kStageBytes + wave * 1024, src.x, src.y);
+    gload_lds4(stat_arr + base + min(i0 + lane, p.Sq - 1), ldl0 + (stage * 128 + (wave & 1) * 64) * 4);
   };
 
   // stationary B operands: Khat and V' rows of this lane's key

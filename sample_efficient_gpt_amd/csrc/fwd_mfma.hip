@@ -62,7 +62,8 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
   __shared__ __attribute__((aligned(1024))) char lds[NS * kStageBytes];
   __shared__ __attribute__((aligned(16))) float gsm[D];  // sm_scale*log2e * g_q * g_k, read as float4 slices
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: everything derived from it stays scalar
   const int ln = lane & 31, hh = lane >> 5;
   const int rep = p.H / p.Hkv;
   const int n_qt = (p.Sq + BQ - 1) / BQ;
@@ -82,7 +83,7 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
 
   const uint32_t lds0 = lds_addr_of(lds);
   const int2 src = swz_src<D>(lane, wave);
-  const uint32_t wave_dst = lds0 + __builtin_amdgcn_readfirstlane(wave) * 1024;
+  const uint32_t wave_dst = lds0 + wave * 1024;
   auto issue_tile = [&](int jt) {  // tile jt -> stage jt % NS
     issue_tile_pair<D>(kbase + (int64_t)jt * kBK * kstep, kstep, vbase + (int64_t)jt * kBK * vstep, vstep,
                        p.Sk - jt * kBK, wave_dst + (jt % NS) * kStageBytes, src.x, src.y);
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
   // One 32-key block.  MASKED / BOUNDED are compile-time so that a whole block is one straight-line
   // scheduling region (a branch in the middle would keep the compiler from interleaving the exp2 work with
   // the neighbouring MFMAs and LDS reads).
-  auto step = [&](auto masked_c, auto bounded_c, uint32_t tr, int kb, int jb, bool more, uint32_t next_rm, int next_kb) {
+  auto step = [&](auto masked_c, auto bounded_c, uint32_t tr, int kb, int jb, uint32_t next_rm, int next_kb) {
     constexpr bool MASKED = decltype(masked_c)::value != 0, BOUNDED = decltype(bounded_c)::value != 0;
     f32x16 s[NQB];
 #pragma unroll
@@ -204,7 +205,7 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
       pb[0][nb] = pack_c_half_sum(s[nb], 0, l_run[nb]);
       pb[1][nb] = pack_c_half_sum(s[nb], 1, l_run[nb]);
     }
-    if (more) request_rowmajor(next_rm, next_kb);
+    request_rowmajor(next_rm, next_kb);  // unconditional: past the last block the fragments are simply unused
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
@@ -233,21 +234,29 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
     __syncthreads();
     if (n_act > 0) request_rowmajor(rm_lane, 0);
     int stage = 0;
-    for (int jt = 0; jt < n_kt; ++jt) {
+    // Two loops instead of a per-block choice inside one: each body is then a single straight-line region
+    // with one variant of the block (a join of the two variants costs a copy of every accumulator).
+    // Loop A: tiles whose two blocks need no mask.  Loop B: the rest (masking a fully visible block is a no-op).
+    const int n_a = n_full / 2;  // n_full <= n_act, so these tiles are all active
+    int jt = 0;
+    for (; jt < n_a; ++jt) {
       const int nstage = stage == NS - 1 ? 0 : stage + 1;
       const bool issued = jt + NS - 1 < n_kt;
       if (issued) issue_tile(jt + NS - 1);
       const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
-      const uint32_t rm_next = rm_lane + nstage * kStageBytes;
-      const int blk = 2 * jt;
-      if (blk < n_act) {
-        if (blk < n_full) step(IC<0>{}, bounded_c, tr, 0, 32 * blk, blk + 1 < n_act, rm, 1);
-        else step(IC<1>{}, bounded_c, tr, 0, 32 * blk, blk + 1 < n_act, rm, 1);
-      }
-      if (blk + 1 < n_act) {
-        if (blk + 1 < n_full) step(IC<0>{}, bounded_c, tr, 1, 32 * blk + 32, blk + 2 < n_act, rm_next, 0);
-        else step(IC<1>{}, bounded_c, tr, 1, 32 * blk + 32, blk + 2 < n_act, rm_next, 0);
-      }
+      step(IC<0>{}, bounded_c, tr, 0, 64 * jt, rm, 1);
+      step(IC<0>{}, bounded_c, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
+      if (issued) wait_vmcnt<(NS - 3) * kLoadsPerTile>(); else wait_vmcnt<0>();
+      __syncthreads();
+      stage = nstage;
+    }
+    for (; jt < n_kt; ++jt) {
+      const int nstage = stage == NS - 1 ? 0 : stage + 1;
+      const bool issued = jt + NS - 1 < n_kt;
+      if (issued) issue_tile(jt + NS - 1);
+      const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
+      if (2 * jt < n_act) step(IC<1>{}, bounded_c, tr, 0, 64 * jt, rm, 1);
+      if (2 * jt + 1 < n_act) step(IC<1>{}, bounded_c, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
       if (issued) wait_vmcnt<(NS - 3) * kLoadsPerTile>(); else wait_vmcnt<0>();
       __syncthreads();
       stage = nstage;
