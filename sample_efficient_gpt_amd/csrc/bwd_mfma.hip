@@ -164,7 +164,9 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   };
   // one 32-key block: tr = lane address inside the block's stage; `more`: a block follows, its row-major
   // fragments start at next_rm
-  auto step = [&](uint32_t tr, int kb, int jb, bool more, uint32_t next_rm, int next_kb) {
+  // MASKED is compile-time so that a whole block is one straight-line scheduling region
+  auto step = [&](auto masked_c, uint32_t tr, int kb, int jb, uint32_t next_rm, int next_kb) {
+    constexpr bool MASKED = decltype(masked_c)::value != 0;
     f32x16 s = c_lse, dpv = c_del;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -177,7 +179,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
       kT[mb][0] = swz_frag_tr<D>(tr, mb, 2 * kb);
       kT[mb][1] = swz_frag_tr<D>(tr, mb, 2 * kb + 1);
     }
-    if ((p.causal && jb + 31 > qw0 + p.q_start) || jb + 32 > p.Sk) {  // block touches the diagonal or the end of the keys
+    if (MASKED) {  // block touches the diagonal or the end of the keys
       // register r holds key jb + 4hh + c_r, c_r = 8(r/4) + r%4: masked iff c_r > qlim - jb - 4hh
       const int t = qlim - jb - 4 * hh;
 #pragma unroll
@@ -187,7 +189,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = fast_exp2(s[r]) * dpv[r];
     const bf16x8 ds0 = pack_c_half(s, 0), ds1 = pack_c_half(s, 1);
-    if (more) request_rowmajor(next_rm, next_kb);
+    request_rowmajor(next_rm, next_kb);  // unconditional: past the last block the fragments are simply unused
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       acc[mb] = mfma32(kT[mb][0], ds0, acc[mb]);
@@ -204,15 +206,29 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   if (n_kt > 2) wait_vmcnt<kLoadsPerTile>(); else wait_vmcnt<0>();  // tiles 0 and 1 have landed
   __syncthreads();
   if (n_act > 0) request_rowmajor(rm_lane, 0);
-  int stage = 0;
-  for (int jt = 0; jt < n_kt; ++jt) {
+  // leading blocks of this wave that need no mask (every key visible to every query of the wave, inside Sk)
+  int n_full = p.Sk / 32;
+  if (p.causal) n_full = min(n_full, (qw0 + p.q_start + 1) / 32);
+  // Loop A: tiles whose two blocks need no mask; loop B: the rest (masking a fully visible block is a no-op).
+  // Two loops, so that each body holds one variant of the block and the accumulators never meet at a join.
+  const int n_a = n_full / 2;  // n_full <= n_act
+  int stage = 0, jt = 0;
+  for (; jt < n_a; ++jt) {
     const int nstage = stage == kStages - 1 ? 0 : stage + 1;
     const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
-    const uint32_t rm_next = rm_lane + nstage * kStageBytes;
-    if (2 * jt < n_act) step(tr, 0, 64 * jt, 2 * jt + 1 < n_act, rm, 1);
-    if (2 * jt + 1 < n_act) step(tr, 1, 64 * jt + 32, 2 * jt + 2 < n_act, rm_next, 0);
+    step(IC<0>{}, tr, 0, 64 * jt, rm, 1);
+    step(IC<0>{}, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
     // stage (jt+3) % 4 == (jt-1) % 4 was last read in the previous iteration: refill it, then make sure
     // this wave's part of tile jt+2 (needed from the next iteration's prefetch on) has landed
+    if (jt + 3 < n_kt) { issue_tile(jt + 3); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
+    __syncthreads();
+    stage = nstage;
+  }
+  for (; jt < n_kt; ++jt) {
+    const int nstage = stage == kStages - 1 ? 0 : stage + 1;
+    const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
+    if (2 * jt < n_act) step(IC<1>{}, tr, 0, 64 * jt, rm, 1);
+    if (2 * jt + 1 < n_act) step(IC<1>{}, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
     if (jt + 3 < n_kt) { issue_tile(jt + 3); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
     __syncthreads();
     stage = nstage;
@@ -350,8 +366,10 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     }
   };
   // one 32-query block (qb = 0/1, compile-time) of the tile whose stage the pointers address;
-  // ib = first query of the block; `more`: a block follows, its row-major fragments start at next_rm
-  auto step = [&](uint32_t tr, uint32_t st, int qb, int ib, bool more, uint32_t next_rm, int next_qb) {
+  // ib = first query of the block; the row-major fragments of the block after it start at next_rm.
+  // MASKED is compile-time so that a whole block is one straight-line scheduling region.
+  auto step = [&](auto masked_c, uint32_t tr, uint32_t st, int qb, int ib, uint32_t next_rm, int next_qb) {
+    constexpr bool MASKED = decltype(masked_c)::value != 0;
     // accumulators of S and dP start from -lse2 / -delta of the 16 query rows their registers map to
     f32x16 s, dpv;
 #pragma unroll
@@ -374,7 +392,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
       dT[mb][1] = swz_frag_tr<D>(tr + Z::kTileBytes, mb, 2 * qb + 1);
       qT[mb][1] = swz_frag_tr<D>(tr, mb, 2 * qb + 1);
     }
-    if ((p.causal && kw0 + 31 > ib + p.q_start) || ib + 32 > p.Sq) {  // block touches the diagonal or the end of the queries
+    if (MASKED) {  // block touches the diagonal or the end of the queries
       // register r holds query ib + 4hh + c_r with c_r = 8(r/4) + r%4 a compile-time constant.
       // masked iff key > query + q_start  <=>  c_r < key - q_start - ib - 4hh,   or query >= Sq
       const int t = p.causal ? key - p.q_start - ib - 4 * hh : -1;
@@ -392,7 +410,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     }
     const bf16x8 p0 = pack_c_half(s, 0), p1 = pack_c_half(s, 1);
     const bf16x8 ds0 = pack_c_half(dpv, 0), ds1 = pack_c_half(dpv, 1);
-    if (more) request_rowmajor(next_rm, next_qb);
+    request_rowmajor(next_rm, next_qb);  // unconditional: past the last block the fragments are simply unused
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       dvacc[mb] = mfma32(dT[mb][0], p0, dvacc[mb]);
@@ -413,18 +431,31 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   if (n_it > 2) wait_vmcnt<kLoadsPerTile>(); else wait_vmcnt<0>();
   __syncthreads();
   if (n_it > 0) request_rowmajor(rm_lane, 0);
-  int stage = 0;
-  for (int it = 0; it < n_it; ++it) {
-    const int nstage = stage == kStages - 1 ? 0 : stage + 1;
-    const int hq = it / n_vis;
-    const int i0 = (qt_start + it - hq * n_vis) * kBK;
-    const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
-    const uint32_t st = st_lane + stage * 512;
-    step(tr, st, 0, i0, true, rm, 1);
-    step(tr, st, 1, i0 + 32, it + 1 < n_it, rm_lane + nstage * kStageBytes, 0);
-    if (it + 3 < n_it) { issue_tile(it + 3); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
-    __syncthreads();
-    stage = nstage;
+  // Per head the visible query tiles t = 0 .. n_vis-1 (first query (qt_start + t) * 64) fall into three runs for
+  // this wave: [0, t_diag) touch the causal diagonal, [t_diag, t_end) need no mask, [t_end, n_vis) run past Sq.
+  // Each run is its own loop so that a loop body holds one variant of the block (whole-block scheduling
+  // regions, no accumulator copies at joins).
+  int t_diag = 0;
+  if (p.causal) t_diag = min(max((max(kw0 + 31 - p.q_start, 0) + kBK - 1) / kBK - qt_start, 0), n_vis);
+  const int t_end = min(max(p.Sq / kBK - qt_start, t_diag), n_vis);
+  int stage = 0, it = 0;
+  auto run_tiles = [&](auto masked_c, int t_lo, int t_hi) {
+    for (int t = t_lo; t < t_hi; ++t, ++it) {
+      const int nstage = stage == kStages - 1 ? 0 : stage + 1;
+      const int i0 = (qt_start + t) * kBK;
+      const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
+      const uint32_t st = st_lane + stage * 512;
+      step(masked_c, tr, st, 0, i0, rm, 1);
+      step(masked_c, tr, st, 1, i0 + 32, rm_lane + nstage * kStageBytes, 0);
+      if (it + 3 < n_it) { issue_tile(it + 3); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
+      __syncthreads();
+      stage = nstage;
+    }
+  };
+  for (int hq = 0; hq < rep; ++hq) {
+    run_tiles(IC<1>{}, 0, t_diag);
+    run_tiles(IC<0>{}, t_diag, t_end);
+    run_tiles(IC<1>{}, t_end, n_vis);
   }
 
   // ---- epilogue: lane = key row, registers = head-dim entries
