@@ -80,8 +80,10 @@ extern "C" {
                                     fp32: delta = rowsum(dY*Y), dgate and the gate-scaled dO            */
 #define SEGPT_BWD_STAGE_DQ 1     /* dQ and the per-workgroup partials of the scale gradient; on the bf16
                                     path also delta, dgate, Qhat and the gate-scaled dO for stage 2      */
-#define SEGPT_BWD_STAGE_DKDV 2   /* dK, dV (, dV_first, partial sums of d vr_coef)                       */
-#define SEGPT_BWD_STAGE_REDUCE 3 /* dg_q, dg_k, d vr_coef from the partials                              */
+#define SEGPT_BWD_STAGE_DKDV 2   /* dK, dV (, dV_first, partial sums of d vr_coef); bf16: also dg_q, dg_k from
+                                    the partials of stage 1                                              */
+#define SEGPT_BWD_STAGE_REDUCE 3 /* d vr_coef from the partials (fp32: also dg_q, dg_k); launches nothing on
+                                    the bf16 path without a value residual                               */
 
 /* [B, heads, S, D] tensor view; the D axis is contiguous (stride 1). Strides in ELEMENTS.
  * The reference's `(h b) S D` flatten (attention.py:199) is stride_b = S*D, stride_h = B*S*D;

@@ -302,7 +302,15 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   const int ln = lane & 31, hh = lane >> 5;
   const int rep = p.H / p.Hkv;
   const int n_kvt = (p.Sk + BKV - 1) / BKV;
-  WgCoord wg = decode_wg(blockIdx.x, n_kvt, p.B, p.Hkv, 1);
+  // Workgroup 0 is an extra one: dispatched first, it only folds the dQ kernel's per-workgroup partials of the
+  // scale-vector gradient (complete: that kernel ran before this one on the stream) while the others compute.
+  if (blockIdx.x == 0) {
+    float* red = reinterpret_cast<float*>(lds);
+    reduce_scale_grad<kThreadsM>(a, tid, red, red + kThreadsM);
+    return;
+  }
+  const int bid = blockIdx.x - 1;  // still a fixed rotation of the hardware's round-robin over the XCDs
+  WgCoord wg = decode_wg(bid, n_kvt, p.B, p.Hkv, 1);
   wg.tile = n_kvt - 1 - wg.tile;  // early key tiles see the most queries: issue them first
   const int b = wg.b, g = wg.g;
   const int k0 = wg.tile * BKV;
@@ -493,7 +501,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     for (int o = 1; o < 64; o <<= 1) { s1 += __shfl_xor(s1, o, 64); s2 += __shfl_xor(s2, o, 64); }
     if (lane == 0) { red[wave * 2] = s1; red[wave * 2 + 1] = s2; }
     __syncthreads();
-    if (tid < 2) a.dcoef_part[(int64_t)blockIdx.x * 2 + tid] = red[tid] + red[2 + tid] + red[4 + tid] + red[6 + tid];
+    if (tid < 2) a.dcoef_part[(int64_t)bid * 2 + tid] = red[tid] + red[2 + tid] + red[4 + tid] + red[6 + tid];
   }
   // dk through the normaliser: W = ln2 * dkacc = dL/dKhat (natural units), dk = b W - (b^3/D)(W.k) k
   {
@@ -525,7 +533,7 @@ template <int D>
 int launch_dkdv_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
   const int n_kvt = (p.Sk + kBwdRows - 1) / kBwdRows;
-  hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D>), dim3((unsigned)(n_kvt * p.Hkv * p.B)), dim3(kThreadsM), 0, st, a);
+  hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D>), dim3((unsigned)(n_kvt * p.Hkv * p.B + 1)), dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 

@@ -94,6 +94,67 @@ __device__ __forceinline__ T* row_ptr_mut(const segpt_tensor4& t, int b, int h, 
 
 __device__ __forceinline__ float sigmoidf_acc(float z) { return 1.0f / (1.0f + expf(-z)); }
 
+// Final reduction of the scale-vector gradient by ONE workgroup of THREADS threads:
+//   tot[d] = sum over the n_dq_blocks partial rows of dg_part[., d]   (fixed order: deterministic)
+//   dg_q = g_k * tot, dg_k = g_q * tot  (summed over d for a scalar parameter)
+// `red` (THREADS floats) and `tot` (D floats) are workgroup-shared scratch.
+template <int THREADS>
+__device__ __forceinline__ void reduce_scale_grad(const KArgs& a, int tid, float* red, float* tot) {
+  const segpt_attn_params& p = a.p;
+  const int D = p.D;
+  const int lanes = THREADS / D;  // threads cooperating on one d
+  const int d = tid % D, sl = tid / D;
+  // eight independent chains hide the load latency
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const float* src = a.dg_part + d;
+  const int n = a.n_dq_blocks;
+  int blk = sl;
+  for (; blk + 7 * lanes < n; blk += 8 * lanes) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(blk + u * lanes) * D];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc[u] += v[u];
+  }
+  for (; blk < n; blk += lanes) acc[0] += src[(int64_t)blk * D];
+  red[tid] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+  __syncthreads();
+  if (tid < D) {
+    float t = 0.f;
+    for (int x = 0; x < lanes; ++x) t += red[x * D + tid];
+    tot[tid] = t;
+  }
+  __syncthreads();
+  if (tid < D) {
+    if (p.gq_numel == D) {
+      const float gk = p.gk_numel == 0 ? 1.f : (p.gk_numel == 1 ? p.g_k[0] : p.g_k[tid]);
+      p.dg_q[tid] = gk * tot[tid];
+    }
+    if (p.gk_numel == D) {
+      const float gq = p.gq_numel == 1 ? p.g_q[0] : p.g_q[tid];
+      p.dg_k[tid] = gq * tot[tid];
+    }
+  }
+  if (tid == 0) {
+    if (p.gq_numel == 1) {
+      float t = 0.f;
+      for (int x = 0; x < D; ++x) {
+        const float gk = p.gk_numel == 0 ? 1.f : (p.gk_numel == 1 ? p.g_k[0] : p.g_k[x]);
+        t += gk * tot[x];
+      }
+      p.dg_q[0] = t;
+    }
+    if (p.gk_numel == 1) {
+      float t = 0.f;
+      for (int x = 0; x < D; ++x) {
+        const float gq = p.gq_numel == 1 ? p.g_q[0] : p.g_q[x];
+        t += gq * tot[x];
+      }
+      p.dg_k[0] = t;
+    }
+  }
+}
+
 // host-side launchers (one per translation unit); each returns a hipError_t as int
 int launch_fwd_f32(const KArgs& a, hipStream_t st);
 int launch_bwd_dkdv_f32(const KArgs& a, hipStream_t st);
@@ -103,7 +164,7 @@ int launch_bwd_dkdv_bf16(const KArgs& a, hipStream_t st);
 int launch_bwd_dq_bf16(const KArgs& a, hipStream_t st);
 int launch_bwd_pre(const KArgs& a, hipStream_t st);     // fp32 path: delta, dgate, do_eff
 int launch_kv_prep(const KArgs& a, hipStream_t st);     // bf16 path: Khat (and V') into kv_workspace
-int launch_bwd_reduce(const KArgs& a, hipStream_t st);  // dg_q, dg_k, dvr_coef from the partials
+int launch_bwd_reduce(const KArgs& a, hipStream_t st);  // fp32: dg_q, dg_k, dvr_coef from the partials; bf16: dvr_coef only
 
 // block counts shared by the workspace carve-up and the launchers
 int dq_blocks(const segpt_attn_params& p);

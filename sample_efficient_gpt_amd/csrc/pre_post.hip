@@ -124,58 +124,8 @@ __global__ __launch_bounds__(kReduceThreads) void bwd_reduce_kernel(KArgs a) {
   __shared__ float red[kReduceThreads];
   __shared__ float tot[128];
   const int tid = threadIdx.x;
-  const int D = p.D;
-  const int lanes = kReduceThreads / D;  // threads cooperating on one d
-  const int d = tid % D, sl = tid / D;
-  // fixed summation order (deterministic); eight independent chains hide the load latency
-  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const float* src = a.dg_part + d;
-  const int n = a.n_dq_blocks;
-  int blk = sl;
-  for (; blk + 7 * lanes < n; blk += 8 * lanes) {
-    float v[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(blk + u * lanes) * D];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) acc[u] += v[u];
-  }
-  for (; blk < n; blk += lanes) acc[0] += src[(int64_t)blk * D];
-  red[tid] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
-  __syncthreads();
-  if (tid < D) {
-    float t = 0.f;
-    for (int x = 0; x < lanes; ++x) t += red[x * D + tid];
-    tot[tid] = t;
-  }
-  __syncthreads();
-  if (tid < D) {
-    if (p.gq_numel == D) {
-      const float gk = p.gk_numel == 0 ? 1.f : (p.gk_numel == 1 ? p.g_k[0] : p.g_k[tid]);
-      p.dg_q[tid] = gk * tot[tid];
-    }
-    if (p.gk_numel == D) {
-      const float gq = p.gq_numel == 1 ? p.g_q[0] : p.g_q[tid];
-      p.dg_k[tid] = gq * tot[tid];
-    }
-  }
-  if (tid == 0) {
-    if (p.gq_numel == 1) {
-      float t = 0.f;
-      for (int x = 0; x < D; ++x) {
-        const float gk = p.gk_numel == 0 ? 1.f : (p.gk_numel == 1 ? p.g_k[0] : p.g_k[x]);
-        t += gk * tot[x];
-      }
-      p.dg_q[0] = t;
-    }
-    if (p.gk_numel == 1) {
-      float t = 0.f;
-      for (int x = 0; x < D; ++x) {
-        const float gq = p.gq_numel == 1 ? p.g_q[0] : p.g_q[x];
-        t += gq * tot[x];
-      }
-      p.dg_k[0] = t;
-    }
-  }
+  // bf16: the scale-vector gradient is reduced inside the dK/dV kernel (by its lightest workgroup)
+  if (p.dtype == SEGPT_DTYPE_FP32) reduce_scale_grad<kReduceThreads>(a, tid, red, tot);
   if (p.vr_coef) {
     __syncthreads();
     float s1 = 0.f, s2 = 0.f;
@@ -234,6 +184,7 @@ int launch_kv_prep(const KArgs& a, hipStream_t st) {
 }
 
 int launch_bwd_reduce(const KArgs& a, hipStream_t st) {
+  if (a.p.dtype == SEGPT_DTYPE_BF16 && !a.p.vr_coef) return 0;  // nothing left to reduce
   hipLaunchKernelGGL(bwd_reduce_kernel, dim3(1), dim3(kReduceThreads), 0, st, a);
   return (int)hipGetLastError();
 }
