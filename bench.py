@@ -32,6 +32,10 @@ if ROOT not in sys.path:
 
 MI355X_BF16_DENSE_TFLOPS = 2516.6  # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz (vendor dense figure, no sparsity)
 MI355X_HBM_GBS = 8000.0
+# HBM bytes per launch (read + write) at cfg 3, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a plain
+# copy kernel of known size (FETCH_SIZE reads 0.5 of the true bytes on this part, WRITE_SIZE 1.0); profiler numbers,
+# not measured by this script
+PMC_TRAFFIC_BYTES_CFG3 = {"fwd": 117.1e6, "bwd_dq": 304.1e6, "bwd_dkdv": 195.0e6}
 
 
 def cpu_baseline(c, batches: int, budget_s: float = 12.0):
@@ -78,6 +82,9 @@ def main():
     ap.add_argument("--cfg", type=int, default=3, help="benchmark configuration (3 = IMU-1 shape fwd+bwd, the headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batches", type=int, default=2)
+    ap.add_argument("--copy-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (a kernel of known traffic, for scaling "
+                         "the profiler's FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU only (the attention path has no cross-GPU step); "
@@ -114,6 +121,12 @@ def main():
                 plan.backward_stage(s, kv_prepared=True)
                 events[2 + s].record()
 
+    if args.copy_mib > 0:
+        src = torch.empty(args.copy_mib << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step_plain()
     # ---- timed region: exactly K steps through segpt_attn_fwd + segpt_attn_bwd
@@ -186,7 +199,7 @@ def main():
             "peak": MI355X_BF16_DENSE_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / MI355X_BF16_DENSE_TFLOPS, 4),
-            "traffic": None,
+            "traffic": PMC_TRAFFIC_BYTES_CFG3.get(dom) if args.cfg == 3 else None,
             "credited_flops_per_launch": credited[dom],
             "avg_launch_ms": round(kern_ms[dom], 5),
             "timing": "HIP events between the stages, second pass over the same K steps",
