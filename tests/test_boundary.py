@@ -193,3 +193,23 @@ def test_input_generators_are_seeded_and_shaped():
     lam = float(x["vr_coef"][0])
     assert 0.3 <= lam <= 0.7 and abs(float(x["vr_coef"].sum()) - 1) < 1e-6
     assert CONFIGS[3].flops() == 7 * 8 * 18 * 2048 * 2048 * 64 and CONFIGS[2].flops() == 2 * 8 * 18 * 2048 * 2048 * 64
+
+
+def test_library_op_is_registered_with_a_shape_only_implementation():
+    """torch.ops.segpt.qknorm_attention: schema, fake (meta) forward and backward shapes, no kernel involved."""
+    from sample_efficient_gpt_amd import qknorm_attention_op
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    assert hasattr(torch.ops.segpt, "qknorm_attention") and hasattr(torch.ops.segpt, "qknorm_attention_backward")
+    mk = lambda *s, dt=torch.bfloat16: torch.empty(*s, dtype=dt, device="meta", requires_grad=True)
+    q, k, v, g = mk(2, 6, 96, 64), mk(2, 2, 96, 64), mk(2, 2, 96, 64), mk(64, dt=torch.float32)
+    y, lse = qknorm_attention_op(q, k, v, g, None, return_lse=True)
+    assert y.shape == q.shape and y.dtype == q.dtype and lse.shape == (2, 6, 96) and lse.dtype == torch.float32
+    y.sum().backward()
+    assert q.grad.shape == q.shape and k.grad.shape == k.shape and v.grad.shape == v.shape and g.grad.shape == g.shape
+    with FakeTensorMode():  # what torch.compile sees: device tensors without storage
+        dev = lambda *s, dt=torch.bfloat16: torch.empty(*s, dtype=dt, device="cuda")
+        out = torch.ops.segpt.qknorm_attention(dev(1, 4, 50, 128), dev(1, 2, 70, 128), dev(1, 2, 70, 128), dev(1, dt=torch.float32),
+                                               None, dev(1, 2, 70, 128), dev(2, dt=torch.float32), dev(1, 50, 4), 2.0, 1e-6, 0.1, True, 20)
+        assert out[0].shape == (1, 4, 50, 128) and out[1].shape == (1, 4, 50)
+        assert out[2].numel() == 2 * (2 * 70 * 128 * 2 + 255) // 256 * 256 or out[2].numel() >= 2 * 2 * 70 * 128 * 2

@@ -218,6 +218,36 @@ def test_plan_reuses_forward_kv_workspace_and_stages_match(gpu_device):
         plan.forward()
 
 
+def test_library_op_compiled_and_checkpointed_matches_eager(gpu_device):
+    """torch.ops.segpt.qknorm_attention under torch.compile (aot_eager: the op stays one opaque node) and under
+    non-reentrant activation checkpointing gives bit-identical outputs and gradients to the autograd Function."""
+    from torch.utils.checkpoint import checkpoint
+
+    from sample_efficient_gpt_amd import qknorm_attention_op
+
+    x = gen(2, 6, 2, 160, 160, 64, BF16, extras=True, seed=21)
+    names = ["q", "k", "v", "g_q", "g_k", "v_first", "vr_coef", "gate_logits"]
+
+    def run(fn):
+        t = {n: x[n].to(gpu_device).requires_grad_(True) for n in names}
+        y = fn(t["q"], t["k"], t["v"], t["g_q"], t["g_k"], v_first=t["v_first"], vr_coef=t["vr_coef"], gate_logits=t["gate_logits"])
+        y.backward(x["d_o"].to(gpu_device))
+        return [y.detach()] + [t[n].grad for n in names]
+
+    print("library op: eager / compiled / checkpointed", flush=True)
+    ref = run(qknorm_attention)
+    eager = run(qknorm_attention_op)
+    compiled = run(torch.compile(qknorm_attention_op, backend="aot_eager", fullgraph=True))
+    ckpt = run(lambda *a, **kw: checkpoint(qknorm_attention_op, *a, use_reentrant=False, **kw))
+    torch.cuda.synchronize()
+    for other in (eager, compiled, ckpt):
+        for a, b in zip(ref, other):
+            assert torch.equal(a, b)
+    torch.library.opcheck(torch.ops.segpt.qknorm_attention,
+                          tuple(x[n].to(gpu_device) for n in names) + (2.0, 1e-6, 0.125, True, 0),
+                          test_utils=("test_schema", "test_faketensor"))
+
+
 def test_backward_is_deterministic(gpu_device):
     x = gen(2, 6, 2, 512, 512, 64, BF16, extras=True, seed=4)
     a = run_gpu(x, gpu_device)
