@@ -76,6 +76,28 @@ def _vec(g, d, like):
     return g
 
 
+# --------------------------------------------------------------------------- rotary embedding (the step before)
+
+
+def rope_tables(max_seq_len: int, theta_base: float, d_k: int, dtype=torch.float64):
+    """cos, sin [max_seq_len, d_k // 2] with angle(pos, j) = pos * theta_base ** (-2 j / d_k).  rope.py:12-24."""
+    j = torch.arange(0, d_k // 2, dtype=dtype)
+    inv_freqs = torch.as_tensor(theta_base, dtype=dtype) ** (-2 * j / d_k)
+    ang = torch.outer(torch.arange(max_seq_len, dtype=dtype), inv_freqs)
+    return ang.cos(), ang.sin()
+
+
+def apply_rope(x, cos, sin, pos0: int = 0):
+    """Split-half rotation of x [..., S, D]: pairs (j, j + D/2); row s uses table row pos0 + s.  rope.py:36-56
+    (the reference computes in fp32 and casts back to the input dtype; here the caller's dtype is kept)."""
+    S, D = x.shape[-2], x.shape[-1]
+    half = D // 2
+    c = cos[pos0 : pos0 + S].to(x.dtype)
+    sn = sin[pos0 : pos0 + S].to(x.dtype)
+    x1, x2 = x[..., :half], x[..., half:]
+    return torch.cat([x1 * c - x2 * sn, x1 * sn + x2 * c], dim=-1)
+
+
 # --------------------------------------------------------------------------- family forward
 
 
@@ -94,12 +116,18 @@ def attention_forward(
     vr_coef=None,
     gate_logits=None,
     gate_scale: float = 2.0,
+    rope=None,
+    rope_q_pos0: int | None = None,
+    rope_k_pos0: int = 0,
 ):
     """Generalised QK-norm attention in canonical layout.
 
     q [B,H,Sq,D]; k, v, v_first [B,Hkv,Sk,D]; g_q, g_k numel 1 or D;
     vr_coef (c1, c2) tensor/sequence; gate_logits [B,Sq,H].
     Query head h reads kv head h // (H // Hkv)  (attention.py:207-218).
+    rope = (cos, sin) tables: q and k are rotated before the normalisation, as the reference's caller does
+    (attention.py:202-204); query row i sits at position rope_q_pos0 + i (default q_start, attention.py:191-195),
+    key row j at rope_k_pos0 + j.
     Computes in the dtype of ``q`` (callers pass fp32 or fp64).
     Returns (y, lse, o_ungated, v_mixed); lse is in natural-log units.
     """
@@ -111,6 +139,9 @@ def attention_forward(
         sm_scale = 1.0 / math.sqrt(D)
     gq = _vec(g_q, D, q)
     gk = _vec(g_k, D, q)
+    if rope is not None:
+        q = apply_rope(q, rope[0], rope[1], q_start if rope_q_pos0 is None else rope_q_pos0)
+        k = apply_rope(k, rope[0], rope[1], rope_k_pos0)
 
     qn = q * rms_inv(q, eps) * gq
     kn = k * rms_inv(k, eps) * gk

@@ -64,6 +64,8 @@ class AttnParams(C.Structure):
         ("workspace_bytes", C.c_size_t),
         ("kv_workspace", C.c_void_p),
         ("kv_workspace_bytes", C.c_size_t),
+        ("rope_cos", C.c_void_p), ("rope_sin", C.c_void_p),
+        ("rope_len", C.c_int32), ("rope_q_pos0", C.c_int32), ("rope_k_pos0", C.c_int32), ("reserved0", C.c_int32),
     ]
 
 

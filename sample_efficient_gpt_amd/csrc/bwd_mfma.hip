@@ -94,16 +94,26 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     const uint16_t* yp = row_ptr<uint16_t>(p.o, b, h, row_c) + 8 * hh;
     const uint16_t* dp = row_ptr<uint16_t>(p.d_o, b, h, row_c) + 8 * hh;
     u32x4 qraw[KS], dyraw[KS];
-    float ss = 0.f, dl = 0.f;
+    float dl = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       qraw[ks] = *reinterpret_cast<const u32x4*>(qp + 16 * ks);
       dyraw[ks] = *reinterpret_cast<const u32x4*>(dp + 16 * ks);
       const u32x4 y = *reinterpret_cast<const u32x4*>(yp + 16 * ks);
-      ss += sumsq8(qraw[ks]);
 #pragma unroll
       for (int i = 0; i < 4; ++i) dl += bf16lo(y[i]) * bf16lo(dyraw[ks][i]) + bf16hi(y[i]) * bf16hi(dyraw[ks][i]);
     }
+    float qx[KS][8];
+    unpack_b_layout<KS>(qraw, qx);
+    if (p.rope_cos) {
+      const int64_t pos = (int64_t)(p.rope_q_pos0 + row_c) * (D / 2);
+      rope_b_layout<KS>(qx, p.rope_cos + pos, p.rope_sin + pos, hh);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) ss += qx[ks][t] * qx[ks][t];
     ss = half_sum(ss);
     delta = half_sum(dl);
     alpha = fast_rsq(ss * (1.0f / D) + p.eps);
@@ -121,10 +131,10 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
       const float4 ga = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh);
       const float4 gb = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh + 4);
       u32x4 w;
-      w[0] = pack_bf16x2(bf16lo(qraw[ks][0]) * f * ga.x, bf16hi(qraw[ks][0]) * f * ga.y);
-      w[1] = pack_bf16x2(bf16lo(qraw[ks][1]) * f * ga.z, bf16hi(qraw[ks][1]) * f * ga.w);
-      w[2] = pack_bf16x2(bf16lo(qraw[ks][2]) * f * gb.x, bf16hi(qraw[ks][2]) * f * gb.y);
-      w[3] = pack_bf16x2(bf16lo(qraw[ks][3]) * f * gb.z, bf16hi(qraw[ks][3]) * f * gb.w);
+      w[0] = pack_bf16x2(qx[ks][0] * f * ga.x, qx[ks][1] * f * ga.y);
+      w[1] = pack_bf16x2(qx[ks][2] * f * ga.z, qx[ks][3] * f * ga.w);
+      w[2] = pack_bf16x2(qx[ks][4] * f * gb.x, qx[ks][5] * f * gb.y);
+      w[3] = pack_bf16x2(qx[ks][6] * f * gb.z, qx[ks][7] * f * gb.w);
       qreg[ks] = as_bf16x8(w);
       if (live) *reinterpret_cast<u32x4*>(a.qhat + ridx * D + 16 * ks + 8 * hh) = w;
       if (p.gate.ptr) {
@@ -238,10 +248,21 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row_c);
   float dot = 0.f;
   float* red = reinterpret_cast<float*>(lds);
+  // q in the C-tile layout (rotated like the operand was), then dq = a (u - (a^2/D)(u.q) q) in the rotated frame
+  // and back through the transpose of the rotation
   float qv[MB][16];
 #pragma unroll
+  for (int mb = 0; mb < MB; ++mb) load_ct_block(qp, mb, hh, qv[mb]);
+  const float* cosr = nullptr;
+  const float* sinr = nullptr;
+  if (p.rope_cos) {
+    const int64_t pos = (int64_t)(p.rope_q_pos0 + row_c) * (D / 2);
+    cosr = p.rope_cos + pos;
+    sinr = p.rope_sin + pos;
+    rope_ct_layout<MB, false>(qv, cosr, sinr, hh);
+  }
+#pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    load_ct_block(qp, mb, hh, qv[mb]);
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int d0 = 32 * mb + 8 * c + 4 * hh;
@@ -260,13 +281,14 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   dot = half_sum(dot);
   const float a3 = alpha * alpha * alpha * (1.0f / D) * dot;
   uint16_t* op = row_ptr_mut<uint16_t>(p.dq, b, h, row_c);
+  float val[MB][16];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    float val[16];
+  for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) val[r] = alpha * acc[mb][r] - a3 * qv[mb][r];
-    store_ct_block(op, mb, hh, live, val);
-  }
+    for (int r = 0; r < 16; ++r) val[mb][r] = alpha * acc[mb][r] - a3 * qv[mb][r];
+  if (p.rope_cos) rope_ct_layout<MB, true>(val, cosr, sinr, hh);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) store_ct_block(op, mb, hh, live, val[mb]);
   // workgroup partial of dg: column sums over the 128 (wave, lane%32) rows, in two levels so that all
   // 256 threads share the LDS reads (fixed order: deterministic)
   __syncthreads();
@@ -507,25 +529,34 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   {
     const uint16_t* kp = row_ptr<uint16_t>(p.k, b, g, key_c);
     float kv[MB][16];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) load_ct_block(kp, mb, hh, kv[mb]);
+    const float* cosr = nullptr;
+    const float* sinr = nullptr;
+    if (p.rope_cos) {  // the normaliser acted on the rotated key: work in that frame, rotate the gradient back
+      const int64_t pos = (int64_t)(p.rope_k_pos0 + key_c) * (D / 2);
+      cosr = p.rope_cos + pos;
+      sinr = p.rope_sin + pos;
+      rope_ct_layout<MB, false>(kv, cosr, sinr, hh);
+    }
     float dot = 0.f, ss = 0.f;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      load_ct_block(kp, mb, hh, kv[mb]);
+    for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) { dot += dkacc[mb][r] * kv[mb][r]; ss += kv[mb][r] * kv[mb][r]; }
-    }
     dot = half_sum(dot) * kLn2;
     ss = half_sum(ss);
     const float beta = fast_rsq(ss * (1.0f / D) + p.eps);
     const float b3 = beta * beta * beta * (1.0f / D) * dot;
     uint16_t* okp = row_ptr_mut<uint16_t>(p.dk, b, g, key_c);
+    float val[MB][16];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      float val[16];
+    for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) val[r] = beta * kLn2 * dkacc[mb][r] - b3 * kv[mb][r];
-      store_ct_block(okp, mb, hh, live, val);
-    }
+      for (int r = 0; r < 16; ++r) val[mb][r] = beta * kLn2 * dkacc[mb][r] - b3 * kv[mb][r];
+    if (p.rope_cos) rope_ct_layout<MB, true>(val, cosr, sinr, hh);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) store_ct_block(okp, mb, hh, live, val[mb]);
   }
 }
 

@@ -92,6 +92,19 @@ __device__ __forceinline__ T* row_ptr_mut(const segpt_tensor4& t, int b, int h, 
   return reinterpret_cast<T*>(t.ptr) + (int64_t)b * t.stride_b + (int64_t)h * t.stride_h + (int64_t)s * t.stride_s;
 }
 
+// Rotary embedding of one split-half pair (x1 = element j, x2 = element j + D/2), rope.py:50-55, and its
+// transpose (the gradient with respect to the unrotated pair).
+__device__ __forceinline__ void rope_pair(float& x1, float& x2, float c, float s) {
+  const float a = x1, b = x2;
+  x1 = a * c - b * s;
+  x2 = a * s + b * c;
+}
+__device__ __forceinline__ void rope_pair_inv(float& x1, float& x2, float c, float s) {
+  const float a = x1, b = x2;
+  x1 = a * c + b * s;
+  x2 = b * c - a * s;
+}
+
 __device__ __forceinline__ float sigmoidf_acc(float z) { return 1.0f / (1.0f + expf(-z)); }
 
 // Final reduction of the scale-vector gradient by ONE workgroup of THREADS threads:

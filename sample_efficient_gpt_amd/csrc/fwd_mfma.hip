@@ -98,12 +98,19 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
     const int row = min(qw0 + 32 * nb + ln, p.Sq - 1);
     const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row) + 8 * hh;
     u32x4 raw[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const u32x4*>(qp + 16 * ks);
+    float x[KS][8];
+    unpack_b_layout<KS>(raw, x);
+    if (p.rope_cos) {
+      const int64_t pos = (int64_t)(p.rope_q_pos0 + row) * (D / 2);
+      rope_b_layout<KS>(x, p.rope_cos + pos, p.rope_sin + pos, hh);
+    }
     float ss = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      raw[ks] = *reinterpret_cast<const u32x4*>(qp + 16 * ks);
-      ss += sumsq8(raw[ks]);
-    }
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) ss += x[ks][t] * x[ks][t];
     ss = half_sum(ss);
     const float alpha = fast_rsq(ss * (1.0f / D) + p.eps);
 #pragma unroll
@@ -111,10 +118,10 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
       const float4 ga = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh);
       const float4 gb = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh + 4);
       u32x4 w;
-      w[0] = pack_bf16x2(bf16lo(raw[ks][0]) * alpha * ga.x, bf16hi(raw[ks][0]) * alpha * ga.y);
-      w[1] = pack_bf16x2(bf16lo(raw[ks][1]) * alpha * ga.z, bf16hi(raw[ks][1]) * alpha * ga.w);
-      w[2] = pack_bf16x2(bf16lo(raw[ks][2]) * alpha * gb.x, bf16hi(raw[ks][2]) * alpha * gb.y);
-      w[3] = pack_bf16x2(bf16lo(raw[ks][3]) * alpha * gb.z, bf16hi(raw[ks][3]) * alpha * gb.w);
+      w[0] = pack_bf16x2(x[ks][0] * alpha * ga.x, x[ks][1] * alpha * ga.y);
+      w[1] = pack_bf16x2(x[ks][2] * alpha * ga.z, x[ks][3] * alpha * ga.w);
+      w[2] = pack_bf16x2(x[ks][4] * alpha * gb.x, x[ks][5] * alpha * gb.y);
+      w[3] = pack_bf16x2(x[ks][6] * alpha * gb.z, x[ks][7] * alpha * gb.w);
       qreg[nb][ks] = as_bf16x8(w);
     }
   }

@@ -210,6 +210,50 @@ __device__ __forceinline__ bf16x8 pack_c_half_sum(const f32x16& c, int s, float&
   return as_bf16x8(w);
 }
 
+// ---- rotary embedding in the two register layouts of a tensor row (cosr / sinr: the table row of the
+// row's position, D/2 floats; both NULL-free: callers test p.rope_cos first)
+// B-operand layout: x[ks][t] = element 16 ks + 8 hh + t; the partner of ks is ks + KS/2 in the same lane
+template <int KS>
+__device__ __forceinline__ void rope_b_layout(float (&x)[KS][8], const float* cosr, const float* sinr, int hh) {
+#pragma unroll
+  for (int ks = 0; ks < KS / 2; ++ks) {
+    const float4 c0 = *reinterpret_cast<const float4*>(cosr + 16 * ks + 8 * hh);
+    const float4 c1 = *reinterpret_cast<const float4*>(cosr + 16 * ks + 8 * hh + 4);
+    const float4 s0 = *reinterpret_cast<const float4*>(sinr + 16 * ks + 8 * hh);
+    const float4 s1 = *reinterpret_cast<const float4*>(sinr + 16 * ks + 8 * hh + 4);
+    const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+    const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+    for (int t = 0; t < 8; ++t) rope_pair(x[ks][t], x[ks + KS / 2][t], c[t], sn[t]);
+  }
+}
+// C-tile layout of load_ct_block / store_ct_block: x[mb][4c + i] = element 32 mb + 8 c + 4 hh + i; the
+// partner of mb is mb + MB/2 in the same lane and register
+template <int MB, bool INVERSE>
+__device__ __forceinline__ void rope_ct_layout(float (&x)[MB][16], const float* cosr, const float* sinr, int hh) {
+#pragma unroll
+  for (int mb = 0; mb < MB / 2; ++mb)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float4 c4 = *reinterpret_cast<const float4*>(cosr + 32 * mb + 8 * c + 4 * hh);
+      const float4 s4 = *reinterpret_cast<const float4*>(sinr + 32 * mb + 8 * c + 4 * hh);
+      const float cc[4] = {c4.x, c4.y, c4.z, c4.w}, ss[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (INVERSE) rope_pair_inv(x[mb][4 * c + i], x[mb + MB / 2][4 * c + i], cc[i], ss[i]);
+        else rope_pair(x[mb][4 * c + i], x[mb + MB / 2][4 * c + i], cc[i], ss[i]);
+      }
+    }
+}
+// raw bf16 words of a B-operand row -> floats
+template <int KS>
+__device__ __forceinline__ void unpack_b_layout(const u32x4 (&raw)[KS], float (&x)[KS][8]) {
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { x[ks][2 * i] = bf16lo(raw[ks][i]); x[ks][2 * i + 1] = bf16hi(raw[ks][i]); }
+}
+
 // ---- helpers shared by the ring kernels (forward, dQ, dK/dV)
 __device__ __forceinline__ float gprod_at(const segpt_attn_params& p, int d) {
   float g = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];

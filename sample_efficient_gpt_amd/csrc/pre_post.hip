@@ -97,6 +97,18 @@ __global__ __launch_bounds__(256) void kv_prep_kernel(KArgs a) {
   const int b = (int)(r / ((int64_t)p.Sk * p.Hkv));
   float k[8];
   Elem<uint16_t>::load(row_ptr<uint16_t>(p.k, b, g, s) + part * 8, k);
+  if (p.rope_cos) {
+    // split-half pairs (j, j + D/2): the partner element sits TPR/2 lanes away, same slot
+    const int jp = (part % (TPR / 2)) * 8;
+    const float* cr = p.rope_cos + (int64_t)(p.rope_k_pos0 + s) * (D / 2) + jp;
+    const float* sr = p.rope_sin + (int64_t)(p.rope_k_pos0 + s) * (D / 2) + jp;
+    const bool first = part < TPR / 2;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float other = __shfl_xor(k[e], TPR / 2, 64);
+      k[e] = first ? k[e] * cr[e] - other * sr[e] : other * sr[e] + k[e] * cr[e];
+    }
+  }
   float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) ss += k[e] * k[e];

@@ -35,7 +35,21 @@ def _scale_arg(g, device):
     return g.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
 
 
-def _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start):
+def _rope_arg(rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, q_start, device, head_dim):
+    """Normalise the rotary-embedding arguments to `(cos, sin, q_pos0, k_pos0)` (fp32 contiguous device tables
+    of shape [len, head_dim // 2]) or None.  Query row i sits at position q_pos0 + i (default: q_start, as in
+    the reference's caller, attention.py:191-204), key row j at k_pos0 + j."""
+    if rope_cos is None and rope_sin is None:
+        return None
+    assert rope_cos is not None and rope_sin is not None, "rope_cos and rope_sin go together"
+    cos = rope_cos.detach().to(device=device, dtype=torch.float32).contiguous()
+    sin = rope_sin.detach().to(device=device, dtype=torch.float32).contiguous()
+    assert cos.dim() == 2 and cos.shape == sin.shape and cos.shape[1] == head_dim // 2, "rope tables must be [len, head_dim // 2]"
+    return cos, sin, int(q_start if rope_q_pos0 is None else rope_q_pos0), int(rope_k_pos0)
+
+
+def _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start,
+                 rope=None):
     B, H, Sq, D = q.shape
     p.dtype = _DTYPES[q.dtype]
     p.B, p.H, p.Hkv, p.Sq, p.Sk, p.D = B, H, k.shape[1], Sq, k.shape[2], D
@@ -49,6 +63,10 @@ def _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scal
     p.gate = _lib.t3(gate)
     p.lse = _lib.ptr(lse)
     p.g_q, p.g_k, p.vr_coef = _lib.ptr(g_q), _lib.ptr(g_k), _lib.ptr(vr_coef)
+    if rope is not None:
+        cos, sin, q_pos0, k_pos0 = rope
+        p.rope_cos, p.rope_sin, p.rope_len = cos.data_ptr(), sin.data_ptr(), cos.shape[0]
+        p.rope_q_pos0, p.rope_k_pos0 = q_pos0, k_pos0
 
 
 def _check_inputs(q, k, v, g_q, g_k, v_first, vr_coef, gate):
@@ -70,14 +88,14 @@ def _check_inputs(q, k, v, g_q, g_k, v_first, vr_coef, gate):
         assert gate.shape == (B, Sq, H), "gate_logits must be [B, Sq, H]"
 
 
-def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y):
+def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope=None):
     """Launch the forward on canonical 4-D views; returns (lse [B,H,Sq] fp32, kv workspace).  `y` is written.
     The kv workspace holds the normalised keys (and mixed values) the backward can reuse."""
     lib = _lib.load()
     B, H, Sq, _ = q.shape
     lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
     p = _lib.new_params()
-    _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start)
+    _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope)
     kv_ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_KV, q.device)
     p.kv_workspace, p.kv_workspace_bytes = kv_ws.data_ptr(), kv_ws.numel()
     rc = lib.segpt_attn_fwd(p, torch.cuda.current_stream(q.device).cuda_stream)
@@ -87,7 +105,7 @@ def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scal
 
 
 def _backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y, lse, dy,
-              dq, dk, dv, dv_first, dgate, kv_ws=None):
+              dq, dk, dv, dv_first, dgate, kv_ws=None, rope=None):
     """Launch the backward; dq/dk/dv(/dv_first/dgate) are written; returns (dg_q, dg_k, dvr_coef) fp32.
     `kv_ws`: the forward's kv workspace (skips the key/value pre-pass); None allocates a fresh one."""
     lib = _lib.load()
@@ -96,7 +114,7 @@ def _backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_sca
     dg_k = None if g_k is None else torch.empty_like(g_k)
     dcoef = None if vr_coef is None else torch.empty(2, dtype=torch.float32, device=dev)
     p = _lib.new_params()
-    _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start)
+    _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope)
     p.d_o, p.dq, p.dk, p.dv = _lib.t4(dy), _lib.t4(dq), _lib.t4(dk), _lib.t4(dv)
     p.dv_first = _lib.t4(dv_first)
     p.dgate = _lib.t3(dgate)
@@ -122,7 +140,7 @@ class _CoreFunc(torch.autograd.Function):
     """Canonical-layout op: q [B,H,Sq,D], k/v/v_first [B,Hkv,Sk,D], gate [B,Sq,H]."""
 
     @staticmethod
-    def forward(ctx, q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start):
+    def forward(ctx, q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope=None):
         gq32, gk32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device)
         coef32 = None if vr_coef is None else vr_coef.detach().to(device=q.device, dtype=torch.float32).reshape(-1).contiguous()
         _check_inputs(q, k, v, gq32, gk32, v_first, coef32, gate)
@@ -133,17 +151,17 @@ class _CoreFunc(torch.autograd.Function):
         y = torch.empty_like(q)
         if y.stride(-1) != 1:
             y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-        lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y)
+        lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope)
         # the normalised keys (bf16 path) are kept for the backward: 1/rep of q's size
         ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse, kv_ws)
-        ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start)
+        ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start, rope)
         ctx.mark_non_differentiable(lse)
         return y, lse
 
     @staticmethod
     def backward(ctx, dy, _dlse):
         q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse, kv_ws = ctx.saved_tensors
-        gate_scale, eps, sm_scale, causal, q_start = ctx.cfg
+        gate_scale, eps, sm_scale, causal, q_start, rope = ctx.cfg
         gq32, gk32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device)
         coef32 = None if vr_coef is None else vr_coef.detach().to(device=q.device, dtype=torch.float32).reshape(-1).contiguous()
         dy = _lastdim_contig(dy)
@@ -153,24 +171,30 @@ class _CoreFunc(torch.autograd.Function):
         dv_first = None if v_first is None else torch.empty_like(v_first)
         dgate = None if gate is None else torch.empty_like(gate)
         dg_q, dg_k, dcoef = _backward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal,
-                                      q_start, y, lse, dy, dq, dk, dv, dv_first, dgate, kv_ws)
+                                      q_start, y, lse, dy, dq, dk, dv, dv_first, dgate, kv_ws, rope)
         dg_q = dg_q.reshape(g_q.shape).to(g_q.dtype)
         if g_k is not None:
             dg_k = dg_k.reshape(g_k.shape).to(g_k.dtype)
         if vr_coef is not None:
             dcoef = dcoef.reshape(vr_coef.shape).to(vr_coef.dtype)
-        return dq, dk, dv, dg_q, dg_k, dv_first, dcoef, dgate, None, None, None, None, None
+        return dq, dk, dv, dg_q, dg_k, dv_first, dcoef, dgate, None, None, None, None, None, None
 
 
 def qknorm_attention(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate_logits=None, gate_scale=2.0,
-                     eps=1e-6, sm_scale=None, causal=True, q_start=0, return_lse=False):
+                     eps=1e-6, sm_scale=None, causal=True, q_start=0, return_lse=False,
+                     rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0):
     """Fused QK-norm attention on canonical views.
 
     q ``[B,H,Sq,D]``; k, v, v_first ``[B,Hkv,Sk,D]`` (any strides, last dim contiguous, rows 16 B
     aligned); g_q, g_k scale parameters of 1 or D elements; vr_coef device tensor ``[2]`` = (c1, c2)
     with ``v' = c1 v + c2 v_first``; gate_logits ``[B,Sq,H]`` with ``y = gate_scale*sigmoid(z)*o``.
+    rope_cos / rope_sin ``[len, D/2]``: q and k are the UNROTATED projections and the split-half rotary
+    embedding (rope.py:36-56) is applied inside the kernels' loads (bf16 only); query row i sits at position
+    ``rope_q_pos0 + i`` (default ``q_start``), key row j at ``rope_k_pos0 + j``.
     """
-    y, lse = _CoreFunc.apply(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start)
+    rope = _rope_arg(rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, q_start, q.device, q.shape[-1])
+    y, lse = _CoreFunc.apply(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
+                             rope)
     return (y, lse) if return_lse else y
 
 
@@ -184,8 +208,9 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
     """Drop-in for ``TritonFlashAttnQKNormFunc`` (triton_flash_attn_qknorm.py:262-343).
 
     ``apply(Q, K, V, gain, is_causal=True, q_start=0, k_gain=None, v_first=None, vr_coef=None,
-    gate_logits=None, gate_scale=2.0, n_kv_heads=None, eps=1e-6, sm_scale=None)`` -- positional only,
-    as autograd Functions are.  ``Q [(h b), Nq, d]``, ``K, V [(h b) or (hkv b), Nk, d]`` contiguous
+    gate_logits=None, gate_scale=2.0, n_kv_heads=None, eps=1e-6, sm_scale=None, rope_cos=None,
+    rope_sin=None)`` -- positional only, as autograd Functions are.  With the rope tables Q and K are the
+    unrotated projections (positions ``q_start + i`` for queries, ``j`` for keys, attention.py:191-204).  ``Q [(h b), Nq, d]``, ``K, V [(h b) or (hkv b), Nk, d]`` contiguous
     device tensors (2-D inputs are promoted to 3-D, the output stays 3-D, :278-281).  When K/V carry
     fewer rows than Q they are un-expanded GQA tensors and ``n_kv_heads`` is required; query row
     ``n = h*B + b`` then reads kv row ``(h // rep)*B + b`` exactly as the reference's
@@ -194,7 +219,8 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, Q, K, V, gain, is_causal=True, q_start=0, k_gain=None, v_first=None, vr_coef=None,
-                gate_logits=None, gate_scale=2.0, n_kv_heads=None, eps=1e-6, sm_scale=None):
+                gate_logits=None, gate_scale=2.0, n_kv_heads=None, eps=1e-6, sm_scale=None, rope_cos=None,
+                rope_sin=None):
         assert Q.is_cuda and Q.is_contiguous()
         assert K.is_cuda and K.is_contiguous()
         assert V.is_cuda and V.is_contiguous()
@@ -224,16 +250,17 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
         if sm_scale is None:
             sm_scale = 1.0 / math.sqrt(Q.shape[-1])
         O = torch.empty_like(Q)
+        rope = _rope_arg(rope_cos, rope_sin, None, 0, q_start, Q.device, Q.shape[-1])
         lse, kv_ws = _forward(q4, k4, v4, gq32, gk32, vf4, coef32, gate_logits, gate_scale, eps, sm_scale, is_causal,
-                              q_start, _canon(O, H))
+                              q_start, _canon(O, H), rope)
         ctx.save_for_backward(lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate_logits, kv_ws)
-        ctx.cfg = (H, Hkv, gate_scale, eps, sm_scale, bool(is_causal), int(q_start))
+        ctx.cfg = (H, Hkv, gate_scale, eps, sm_scale, bool(is_causal), int(q_start), rope)
         return O
 
     @staticmethod
     def backward(ctx, grad_output):
         lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate, kv_ws = ctx.saved_tensors
-        H, Hkv, gate_scale, eps, sm_scale, causal, q_start = ctx.cfg
+        H, Hkv, gate_scale, eps, sm_scale, causal, q_start, rope = ctx.cfg
         grad_output = grad_output.contiguous()
         if grad_output.dtype != Q.dtype:
             grad_output = grad_output.to(Q.dtype)
@@ -248,9 +275,9 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
             _canon(Q, H), _canon(K, Hkv), _canon(V, Hkv), gq32, gk32,
             None if v_first is None else _canon(v_first, Hkv), coef32, gate, gate_scale, eps, sm_scale, causal, q_start,
             _canon(O, H), lse, _canon(grad_output, H), _canon(dQ, H), _canon(dK, Hkv), _canon(dV, Hkv),
-            None if dVf is None else _canon(dVf, Hkv), dgate, kv_ws)
+            None if dVf is None else _canon(dVf, Hkv), dgate, kv_ws, rope)
         dgain = dg_q.reshape(gain.shape).to(gain.dtype)
         dk_gain = None if k_gain is None else dg_k.reshape(k_gain.shape).to(k_gain.dtype)
         dcoef = None if vr_coef is None else dcoef.reshape(vr_coef.shape).to(vr_coef.dtype)
-        #      Q   K   V   gain   causal q_start k_gain  v_first vr_coef gate  gate_scale n_kv eps sm_scale
-        return dQ, dK, dV, dgain, None, None, dk_gain, dVf, dcoef, dgate, None, None, None, None
+        #      Q   K   V   gain   causal q_start k_gain  v_first vr_coef gate  gate_scale n_kv eps sm_scale rope tables
+        return dQ, dK, dV, dgain, None, None, dk_gain, dVf, dcoef, dgate, None, None, None, None, None, None

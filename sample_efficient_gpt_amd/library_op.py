@@ -4,11 +4,12 @@ non-reentrant activation checkpointing (transformer/transformer.py:123-132) as O
 (shape-only) implementation instead of being traced into.
 
     y = torch.ops.segpt.qknorm_attention(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits,
-                                         gate_scale, eps, sm_scale, causal, q_start)[0]
+                                         gate_scale, eps, sm_scale, causal, q_start,
+                                         rope_cos, rope_sin, rope_q_pos0, rope_k_pos0)[0]
 
 or the keyword wrapper ``qknorm_attention_op(...)`` below.  Canonical layout: q ``[B,H,Sq,D]``, k / v /
 v_first ``[B,Hkv,Sk,D]`` (any strides, last dim contiguous), gate_logits ``[B,Sq,H]``; the optional tensors
-are ``None`` when unused.  Returns ``(y, lse, kv_ws)``: the output, the fp32 log-sum-exp ``[B,H,Sq]`` and the
+are ``None`` when unused (rope_q_pos0 = -1 means "q_start").  Returns ``(y, lse, kv_ws)``: the output, the fp32 log-sum-exp ``[B,H,Sq]`` and the
 key/value workspace the backward reuses.  Same kernels and C ABI as ``function.py``; no fallback.
 """
 
@@ -21,7 +22,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .function import _backward, _check_inputs, _forward, _lastdim_contig, _scale_arg
+from .function import _backward, _check_inputs, _forward, _lastdim_contig, _rope_arg, _scale_arg
 
 __all__ = ["qknorm_attention_op"]
 
@@ -33,18 +34,21 @@ def _coef32(vr_coef, device):
 @torch.library.custom_op("segpt::qknorm_attention", mutates_args=())
 def _fwd_op(q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optional[Tensor], v_first: Optional[Tensor],
             vr_coef: Optional[Tensor], gate_logits: Optional[Tensor], gate_scale: float, eps: float, sm_scale: float,
-            causal: bool, q_start: int) -> List[Tensor]:
+            causal: bool, q_start: int, rope_cos: Optional[Tensor], rope_sin: Optional[Tensor],
+            rope_q_pos0: int, rope_k_pos0: int) -> List[Tensor]:
+    rope = _rope_arg(rope_cos, rope_sin, None if rope_q_pos0 < 0 else rope_q_pos0, rope_k_pos0, q_start, q.device, q.shape[-1])
     gq32, gk32, c32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device), _coef32(vr_coef, q.device)
     _check_inputs(q, k, v, gq32, gk32, v_first, c32, gate_logits)
     q, k, v = _lastdim_contig(q), _lastdim_contig(k), _lastdim_contig(v)
     v_first = None if v_first is None else _lastdim_contig(v_first)
     y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, c32, gate_logits, gate_scale, eps, sm_scale, causal, q_start, y)
+    lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, c32, gate_logits, gate_scale, eps, sm_scale, causal, q_start, y, rope)
     return [y, lse, kv_ws]
 
 
 @_fwd_op.register_fake
-def _(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start):
+def _(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
+      rope_cos, rope_sin, rope_q_pos0, rope_k_pos0):
     B, H, Sq, D = q.shape
     y = q.new_empty((B, H, Sq, D))
     lse = q.new_empty((B, H, Sq), dtype=torch.float32)
@@ -59,9 +63,11 @@ def _(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scal
 @torch.library.custom_op("segpt::qknorm_attention_backward", mutates_args=())
 def _bwd_op(dy: Tensor, q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optional[Tensor], v_first: Optional[Tensor],
             vr_coef: Optional[Tensor], gate_logits: Optional[Tensor], y: Tensor, lse: Tensor, kv_ws: Tensor,
-            gate_scale: float, eps: float, sm_scale: float, causal: bool, q_start: int) -> List[Tensor]:
+            gate_scale: float, eps: float, sm_scale: float, causal: bool, q_start: int,
+            rope_cos: Optional[Tensor], rope_sin: Optional[Tensor], rope_q_pos0: int, rope_k_pos0: int) -> List[Tensor]:
     """Returns [dq, dk, dv, dg_q, dg_k, dv_first, dvr_coef, dgate]; absent ones are empty tensors."""
     dev = q.device
+    rope = _rope_arg(rope_cos, rope_sin, None if rope_q_pos0 < 0 else rope_q_pos0, rope_k_pos0, q_start, dev, q.shape[-1])
     gq32, gk32, c32 = _scale_arg(g_q, dev), _scale_arg(g_k, dev), _coef32(vr_coef, dev)
     q, k, v = _lastdim_contig(q), _lastdim_contig(k), _lastdim_contig(v)
     v_first = None if v_first is None else _lastdim_contig(v_first)
@@ -72,7 +78,7 @@ def _bwd_op(dy: Tensor, q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optio
     dvf = None if v_first is None else torch.empty_like(v_first)
     dgate = None if gate_logits is None else torch.empty_like(gate_logits)
     dg_q, dg_k, dcoef = _backward(q, k, v, gq32, gk32, v_first, c32, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
-                                  y, lse, dy, dq, dk, dv, dvf, dgate, kv_ws)
+                                  y, lse, dy, dq, dk, dv, dvf, dgate, kv_ws, rope)
     none = q.new_empty((0,))
     return [dq, dk, dv, dg_q.reshape(g_q.shape).to(g_q.dtype),
             none if g_k is None else dg_k.reshape(g_k.shape).to(g_k.dtype),
@@ -82,7 +88,8 @@ def _bwd_op(dy: Tensor, q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optio
 
 
 @_bwd_op.register_fake
-def _(dy, q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, gate_scale, eps, sm_scale, causal, q_start):
+def _(dy, q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, gate_scale, eps, sm_scale, causal, q_start,
+      rope_cos, rope_sin, rope_q_pos0, rope_k_pos0):
     none = q.new_empty((0,))
     return [torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(g_q),
             none if g_k is None else torch.empty_like(g_k),
@@ -92,30 +99,36 @@ def _(dy, q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, gate_
 
 
 def _setup_context(ctx, inputs, output):
-    q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start = inputs
+    (q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
+     rope_cos, rope_sin, rope_q_pos0, rope_k_pos0) = inputs
     y, lse, kv_ws = output
-    ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws)
-    ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start)
+    ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, rope_cos, rope_sin)
+    ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start, rope_q_pos0, rope_k_pos0)
 
 
 def _autograd_backward(ctx, grads):
     dy = grads[0]
-    q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws = ctx.saved_tensors
-    gate_scale, eps, sm_scale, causal, q_start = ctx.cfg
+    q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, rope_cos, rope_sin = ctx.saved_tensors
+    gate_scale, eps, sm_scale, causal, q_start, rope_q_pos0, rope_k_pos0 = ctx.cfg
     dq, dk, dv, dg_q, dg_k, dvf, dcoef, dgate = torch.ops.segpt.qknorm_attention_backward(
-        dy, q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, gate_scale, eps, sm_scale, causal, q_start)
+        dy, q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, gate_scale, eps, sm_scale, causal, q_start,
+        rope_cos, rope_sin, rope_q_pos0, rope_k_pos0)
     return (dq, dk, dv, dg_q, None if g_k is None else dg_k, None if v_first is None else dvf,
-            None if vr_coef is None else dcoef, None if gate_logits is None else dgate, None, None, None, None, None)
+            None if vr_coef is None else dcoef, None if gate_logits is None else dgate, None, None, None, None, None,
+            None, None, None, None)
 
 
 _fwd_op.register_autograd(_autograd_backward, setup_context=_setup_context)
 
 
 def qknorm_attention_op(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate_logits=None, gate_scale=2.0,
-                        eps=1e-6, sm_scale=None, causal=True, q_start=0, return_lse=False):
+                        eps=1e-6, sm_scale=None, causal=True, q_start=0, return_lse=False,
+                        rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0):
     """Keyword front end of ``torch.ops.segpt.qknorm_attention`` (same arguments as ``qknorm_attention``)."""
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
     y, lse, _ = torch.ops.segpt.qknorm_attention(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, float(gate_scale),
-                                                 float(eps), float(sm_scale), bool(causal), int(q_start))
+                                                 float(eps), float(sm_scale), bool(causal), int(q_start),
+                                                 rope_cos, rope_sin, -1 if rope_q_pos0 is None else int(rope_q_pos0),
+                                                 int(rope_k_pos0))
     return (y, lse) if return_lse else y

@@ -8,14 +8,15 @@ import math
 import torch
 
 from . import _lib
-from .function import _fill_common
+from .function import _fill_common, _rope_arg
 
 
 class AttnPlan:
     """Binds canonical-layout tensors (q [B,H,S,D], k/v [B,Hkv,S,D], ...) once; `forward()`,
     `backward()` and `backward_stage(i)` then only enqueue kernels on the current stream."""
 
-    def __init__(self, x: dict, *, eps=1e-6, sm_scale=None, gate_scale=2.0, causal=True, q_start=0, backward=True):
+    def __init__(self, x: dict, *, eps=1e-6, sm_scale=None, gate_scale=2.0, causal=True, q_start=0, backward=True,
+                 rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0):
         self.lib = _lib.load()
         q, k, v = x["q"], x["k"], x["v"]
         dev = q.device
@@ -28,9 +29,10 @@ class AttnPlan:
             sm_scale = 1.0 / math.sqrt(D)
         self.y = torch.empty_like(q)
         self.lse = torch.empty((B, H, Sq), dtype=torch.float32, device=dev)
+        self.rope = _rope_arg(rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, q_start, dev, D)  # keeps the tables alive
         p = _lib.new_params()
         _fill_common(p, q, k, v, self.y, self.lse, self.g_q, self.g_k, self.v_first, self.coef, self.gate, gate_scale,
-                     eps, sm_scale, causal, q_start)
+                     eps, sm_scale, causal, q_start, self.rope)
         self.kv_ws = _lib.alloc_workspace(self.lib, p, _lib.SEGPT_WS_KV, dev)
         p.kv_workspace, p.kv_workspace_bytes = self.kv_ws.data_ptr(), self.kv_ws.numel()
         self.p = p

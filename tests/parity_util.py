@@ -33,8 +33,19 @@ def gen(B, H, Hkv, Sq, Sk, D, dtype, *, extras=False, scalar_gain=False, no_gk=F
     return x
 
 
+def _split_rope(kw, device=None):
+    """kw may carry rope=(cos, sin) (+ rope_q_pos0 / rope_k_pos0): returns the op's and the oracle's keyword sets."""
+    kw = dict(kw)
+    rope = kw.pop("rope", None)
+    if rope is None:
+        return kw, kw
+    gpu_kw = dict(kw, rope_cos=rope[0].float().to(device) if device is not None else rope[0], rope_sin=rope[1].float().to(device) if device is not None else rope[1])
+    return gpu_kw, dict(kw, rope=rope)
+
+
 def run_gpu(x, device, *, backward=True, **kw):
     """Run the HIP op (and its backward) on `device`; returns CPU tensors."""
+    kw, _ = _split_rope(kw, device)
     names = ["q", "k", "v", "g_q", "g_k", "v_first", "vr_coef", "gate_logits"]
     t = {n: (x[n].to(device).requires_grad_(backward) if x.get(n) is not None else None) for n in names}
     y, lse = qknorm_attention(t["q"], t["k"], t["v"], t["g_q"], t["g_k"], v_first=t["v_first"], vr_coef=t["vr_coef"],
@@ -53,6 +64,7 @@ def run_gpu(x, device, *, backward=True, **kw):
 def run_oracle(x, *, backward=True, odtype=torch.float64, **kw):
     """CPU oracle on the same bits, computed in `odtype`."""
     f = lambda n: None if x.get(n) is None else x[n].to(odtype)
+    _, kw = _split_rope(kw)
     okw = dict(kw)
     if f("v_first") is not None:
         okw.update(v_first=f("v_first"), vr_coef=f("vr_coef"))

@@ -335,3 +335,62 @@ def test_variant_b_reference_backward_form_matches_family():
     assert torch.allclose(ex["dk"][:, 0], dk, atol=1e-10)
     assert torch.allclose(ex["dv"][:, 0], p.transpose(1, 2) @ dO, atol=1e-10)
     assert abs(float(ex["dg_q"].sum() - dg)) < 1e-10
+
+
+# ------------------------------------------------------------------ rotary embedding (rope.py:12-56)
+
+
+def test_rope_tables_closed_form():
+    cos, sin = orc.rope_tables(37, 10000.0, 16)
+    assert cos.shape == sin.shape == (37, 8)
+    assert torch.allclose(cos[0], torch.ones(8, dtype=F64)) and torch.allclose(sin[0], torch.zeros(8, dtype=F64))
+    for pos, j in ((1, 0), (5, 3), (36, 7)):
+        ang = pos * 10000.0 ** (-2 * j / 16)
+        assert abs(float(cos[pos, j]) - math.cos(ang)) < 1e-12 and abs(float(sin[pos, j]) - math.sin(ang)) < 1e-12
+    assert abs(float(cos[9, 0]) - math.cos(9.0)) < 1e-12  # pair 0 turns by one radian per position
+
+
+def test_rope_is_the_complex_rotation_of_split_half_pairs():
+    # independent formulation: z_j = x_j + i x_{j+D/2},  z_j -> z_j * exp(i * angle(pos, j))
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(2, 3, 11, 8, generator=g, dtype=F64)
+    cos, sin = orc.rope_tables(32, 100.0, 8)
+    pos0 = 5
+    got = orc.apply_rope(x, cos, sin, pos0)
+    z = torch.complex(x[..., :4], x[..., 4:])
+    ang = torch.outer(torch.arange(pos0, pos0 + 11, dtype=F64), 100.0 ** (-2 * torch.arange(4, dtype=F64) / 8))
+    zr = z * torch.polar(torch.ones_like(ang), ang)
+    assert torch.allclose(got, torch.cat([zr.real, zr.imag], -1), atol=1e-12)
+    # a rotation: pair norms and hence the row RMS are unchanged; position 0 is the identity
+    assert torch.allclose(got.pow(2).sum(-1), x.pow(2).sum(-1), atol=1e-12)
+    assert torch.allclose(orc.apply_rope(x[..., :1, :], cos, sin, 0), x[..., :1, :], atol=1e-15)
+    # rotating by pos then by -pos (sin -> -sin) restores x
+    assert torch.allclose(orc.apply_rope(got, cos, -sin, pos0), x, atol=1e-12)
+
+
+def test_rope_in_attention_depends_on_relative_positions_only():
+    q, k, v, _, _ = _rand(Sq=20, D=8, seed=5)
+    cos, sin = orc.rope_tables(64, 50.0, 8)
+    y0, l0, _, _ = orc.attention_forward(q, k, v, None, None, rope=(cos, sin))
+    # same relative offsets, every absolute position shifted by 13: logits q_i.k_j are unchanged
+    y1, l1, _, _ = orc.attention_forward(q, k, v, None, None, rope=(cos, sin), rope_q_pos0=13, rope_k_pos0=13)
+    assert torch.allclose(y0, y1, atol=1e-10) and torch.allclose(l0, l1, atol=1e-10)
+    # it is not a no-op, and it equals rotating the inputs by hand
+    y_plain, _, _, _ = orc.attention_forward(q, k, v, None, None)
+    assert (y0 - y_plain).abs().max() > 1e-3
+    y2, _, _, _ = orc.attention_forward(orc.apply_rope(q, cos, sin), orc.apply_rope(k, cos, sin), v, None, None)
+    assert torch.allclose(y0, y2, atol=1e-12)
+    # decode-style suffix: queries 7.. with q_start=7 sit at positions 7.. by default (attention.py:191-195)
+    y3, _, _, _ = orc.attention_forward(q[:, :, 7:], k, v, None, None, q_start=7, rope=(cos, sin))
+    assert torch.allclose(y3, y0[:, :, 7:], atol=1e-10)
+
+
+def test_rope_gradients_by_gradcheck():
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(1, 2, 5, 4, generator=g, dtype=F64, requires_grad=True)
+    k = torch.randn(1, 1, 5, 4, generator=g, dtype=F64, requires_grad=True)
+    v = torch.randn(1, 1, 5, 4, generator=g, dtype=F64, requires_grad=True)
+    gq = (1 + 0.2 * torch.randn(4, generator=g, dtype=F64)).requires_grad_(True)
+    cos, sin = orc.rope_tables(8, 10.0, 4)
+    fn = lambda q, k, v, gq: orc.attention_forward(q, k, v, gq, None, rope=(cos, sin))[0]
+    assert torch.autograd.gradcheck(fn, (q, k, v, gq), eps=1e-6, atol=1e-6)

@@ -244,8 +244,49 @@ def test_library_op_compiled_and_checkpointed_matches_eager(gpu_device):
         for a, b in zip(ref, other):
             assert torch.equal(a, b)
     torch.library.opcheck(torch.ops.segpt.qknorm_attention,
-                          tuple(x[n].to(gpu_device) for n in names) + (2.0, 1e-6, 0.125, True, 0),
+                          tuple(x[n].to(gpu_device) for n in names) + (2.0, 1e-6, 0.125, True, 0, None, None, -1, 0),
                           test_utils=("test_schema", "test_faketensor"))
+
+
+# ------------------------------------------------------------------ rotary embedding fused into the loads
+
+
+@pytest.mark.parametrize(
+    "B,H,Hkv,Sq,Sk,D,kw,gen_kw",
+    [
+        (2, 6, 2, 300, 300, 64, {}, {}),
+        (1, 4, 2, 200, 200, 64, {"gate_scale": 2.0}, {"extras": True, "scalar_gain": True}),
+        (1, 4, 1, 160, 160, 128, {}, {}),
+        (1, 3, 3, 72, 200, 64, {"q_start": 128}, {}),                      # queries at positions 128.. (attention.py:191-195)
+        (1, 2, 1, 96, 96, 64, {"rope_q_pos0": 40, "rope_k_pos0": 40}, {}),  # explicit positions
+        (1, 2, 2, 80, 140, 64, {"causal": False}, {}),
+    ],
+)
+def test_bf16_fused_rope(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
+    """q, k are the unrotated projections; the kernels rotate them in their loads (forward, pre-pass, dQ
+    prologue) and rotate dq, dk back in their epilogues.  Oracle: rope.py's rotation, then the family forward,
+    gradients by autograd (fp64)."""
+    cos, sin = orc.rope_tables(512, 10000.0, D)
+    _case(gpu_device, BF16, B, H, Hkv, Sq, Sk, D, gen_kw=gen_kw, seed=31, rope=(cos, sin), **kw)
+
+
+def test_fused_rope_equals_rotating_first_and_rejects_bad_tables(gpu_device):
+    from sample_efficient_gpt_amd import _lib
+
+    x = gen(1, 4, 2, 256, 256, 64, BF16, seed=33)
+    cos, sin = orc.rope_tables(256, 10000.0, 64)
+    fused = run_gpu(x, gpu_device, backward=False, rope=(cos, sin))
+    # rotate on the host in fp32 and round to bf16 (what the reference's caller hands its kernel)
+    xr = dict(x, q=orc.apply_rope(x["q"].float(), cos, sin).to(BF16), k=orc.apply_rope(x["k"].float(), cos, sin).to(BF16))
+    twostep = run_gpu(xr, gpu_device, backward=False)
+    assert torch.allclose(fused["y"].float(), twostep["y"].float(), atol=2e-2, rtol=1e-2)
+    assert torch.allclose(fused["lse"], twostep["lse"], atol=2e-2, rtol=1e-2)
+    short = orc.rope_tables(100, 10000.0, 64)
+    with pytest.raises(_lib.SegptError):  # table shorter than the positions it must serve
+        run_gpu(x, gpu_device, backward=False, rope=short)
+    xf = gen(1, 2, 2, 64, 64, 64, F32, seed=1)
+    with pytest.raises(_lib.SegptError):  # the fp32 path has no fused rotary embedding
+        run_gpu(xf, gpu_device, backward=False, rope=(cos, sin))
 
 
 def test_backward_is_deterministic(gpu_device):
