@@ -84,6 +84,12 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
                        p.Sk - jt * kBK, wave_dst + (jt % kStages) * kStageBytes, src.x, src.y);
   };
 
+  // start-up tiles first: their latency overlaps the query-row prologue below (vector-memory waits are in
+  // order, so the prologue's own loads complete after them and nothing stays in flight into the loop)
+  issue_tile(0);
+  if (n_kt > 1) issue_tile(1);
+  if (n_kt > 2) issue_tile(2);
+
   // ---- query-row prologue: alpha, Qhat, delta, gate; B operands stay in registers
   if (tid < D) gsm[tid] = gprod_at(p, tid);
   __syncthreads();
@@ -207,13 +213,9 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     }
   };
 
-  // ---- pipeline start-up.  All earlier vector loads are drained first: the tile loads that stay in flight
-  // across iterations must be the youngest vector-memory operations of the wave (waits are in-order).
-  drain_vector_loads();
-  issue_tile(0);
-  if (n_kt > 1) issue_tile(1);
-  if (n_kt > 2) issue_tile(2);
-  if (n_kt > 2) wait_vmcnt<kLoadsPerTile>(); else wait_vmcnt<0>();  // tiles 0 and 1 have landed
+  // ---- pipeline start-up: the tile loads that stay in flight across iterations must be the youngest
+  // vector-memory operations of the wave (waits are in-order); here everything has landed.
+  wait_vmcnt<0>();
   __syncthreads();
   if (n_act > 0) request_rowmajor(rm_lane, 0);
   // leading blocks of this wave that need no mask (every key visible to every query of the wave, inside Sk)
@@ -368,6 +370,11 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     gload_lds4(stat_arr + base + min(i0 + lane, p.Sq - 1), ldl0 + (stage * 128 + (wave & 1) * 64) * 4);
   };
 
+  // start-up tiles first: their latency overlaps the loads of the stationary operands below
+  if (n_it > 0) issue_tile(0);
+  if (n_it > 1) issue_tile(1);
+  if (n_it > 2) issue_tile(2);
+
   // stationary B operands: Khat and V' rows of this lane's key
   bf16x8 kreg[KS], vreg[KS];
   {
@@ -454,11 +461,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   };
 
   // ---- pipeline start-up (see the dQ kernel)
-  drain_vector_loads();
-  if (n_it > 0) issue_tile(0);
-  if (n_it > 1) issue_tile(1);
-  if (n_it > 2) issue_tile(2);
-  if (n_it > 2) wait_vmcnt<kLoadsPerTile>(); else wait_vmcnt<0>();
+  wait_vmcnt<0>();
   __syncthreads();
   if (n_it > 0) request_rowmajor(rm_lane, 0);
   // Per head the visible query tiles t = 0 .. n_vis-1 (first query (qt_start + t) * 64) fall into three runs for

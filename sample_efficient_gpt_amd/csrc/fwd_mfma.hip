@@ -89,6 +89,12 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
                        p.Sk - jt * kBK, wave_dst + (jt % NS) * kStageBytes, src.x, src.y);
   };
 
+  // start-up tiles 0 .. NS-2 first: their latency overlaps the query prologue below (vector-memory waits are
+  // in order, so the prologue's own loads complete after them and nothing stays in flight into the loop)
+#pragma unroll
+  for (int t = 0; t < NS - 1; ++t)
+    if (t < n_kt) issue_tile(t);
+
   // ---- Qhat registers: B operands of S^T, [nb][ks]
   if (tid < D) gsm[tid] = gprod_at(p, tid) * p.sm_scale * kLog2e;
   __syncthreads();
@@ -226,18 +232,14 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
   int n_full = p.Sk / 32;
   if (p.causal) n_full = min(n_full, (qw0 + p.q_start + 1) / 32);
 
-  // ---- pipeline.  All earlier vector loads are drained first: the tile loads that stay in flight across
-  // iterations must be the youngest vector-memory operations of the wave (waits are in-order).
+  // ---- pipeline.  The tile loads that stay in flight across iterations must be the youngest vector-memory
+  // operations of the wave (waits are in-order): everything is complete at the top of the first iteration.
   // Protocol: at the top of iteration jt tiles jt and jt+1 have landed and tiles jt+2 .. jt+NS-2 are in
   // flight; the stage of tile jt-1 is free (everyone passed the barrier that ended iteration jt-1), so tile
   // jt+NS-1 is requested right away and has a whole iteration to land; the wait at the bottom leaves the
   // youngest NS-3 tiles in flight, i.e. tile jt+2 is complete before the barrier.
   auto run = [&](auto bounded_c) {
-    drain_vector_loads();
-#pragma unroll
-    for (int t = 0; t < NS - 1; ++t)
-      if (t < n_kt) issue_tile(t);
-    if (n_kt >= NS - 1) wait_vmcnt<(NS - 3) * kLoadsPerTile>(); else wait_vmcnt<0>();  // tiles 0 and 1 have landed
+    wait_vmcnt<0>();  // the start-up tiles (requested before the query prologue) have landed
     __syncthreads();
     if (n_act > 0) request_rowmajor(rm_lane, 0);
     int stage = 0;

@@ -45,15 +45,6 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float fast_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
-// Wait for every outstanding vector-memory load of this wave and keep the compiler from moving memory
-// operations across this point.  Used once before a pipelined loop: loads that stay in flight ACROSS loop
-// iterations must be the youngest ones, or every in-loop wait for an older load drains them as well.
-__device__ __forceinline__ void drain_vector_loads() {
-  __builtin_amdgcn_sched_barrier(0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt/lgkmcnt untouched
-  __builtin_amdgcn_sched_barrier(0);
-}
-
 // acc + lo + hi of one packed bf16 pair (v_dot2c_f32_bf16 with a (1,1) operand): sums the ROUNDED values,
 // i.e. exactly what the MFMA consuming the packed operand sees.
 __device__ __forceinline__ float add_bf16_pair(uint32_t w, float acc) {
