@@ -74,6 +74,43 @@ def cpu_baseline(c, batches: int, budget_s: float = 12.0):
     }
 
 
+def decode_bench(args):
+    """One generation step: q [B,18,1,64] against k, v [B,6,Sk,64] (bf16), keys normalised on the fly."""
+    import torch
+
+    from sample_efficient_gpt_amd import _lib
+    from sample_efficient_gpt_amd.plan import AttnPlan
+
+    B, H, Hkv, D, Sk = args.decode_batch, 18, 6, 64, args.decode_keys
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(7)
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    x = {"q": mk(B, H, 1, D), "k": mk(B, Hkv, Sk, D), "v": mk(B, Hkv, Sk, D),
+         "g_q": 1.0 + 0.02 * torch.randn(D, generator=g), "g_k": 1.0 + 0.02 * torch.randn(D, generator=g)}
+    plan = AttnPlan(x, q_start=Sk - 1, backward=False)
+    step = lambda: plan.forward(flags=_lib.SEGPT_FLAG_DECODE)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    nbytes = 2 * B * Hkv * Sk * D * 2  # every K and V row once (q, y, partials are < 1 %)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "decode-step attention, K+V bytes per second", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"decode step: B={B} q_heads={H} kv_heads={Hkv} head_dim={D} 1 query against {Sk} cached keys, "
+                               "QK-norm + causal mask, split-key kernels (split + merge launches)"},
+        "roofline": {"kernel": "decode_split_kernel + decode_merge_kernel", "bound": "hbm", "achieved": round(gbs, 1),
+                     "peak": MI355X_HBM_GBS, "unit": "GB/s", "frac": round(gbs / MI355X_HBM_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": nbytes, "timing": "wall clock over the K steps (both launches)"},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -82,6 +119,10 @@ def main():
     ap.add_argument("--cfg", type=int, default=3, help="benchmark configuration (3 = IMU-1 shape fwd+bwd, the headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batches", type=int, default=2)
+    ap.add_argument("--decode-keys", type=int, default=0,
+                    help="instead of a training config: one generation step (1 new token per sequence, IMU-1 heads) "
+                         "against a cache of this many keys, through the split-key decode kernels; reports K+V GB/s")
+    ap.add_argument("--decode-batch", type=int, default=8)
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known traffic, for scaling "
                          "the profiler's FETCH_SIZE / WRITE_SIZE counters)")
@@ -96,6 +137,8 @@ def main():
     from sample_efficient_gpt_amd import CONFIGS, make_inputs
     from sample_efficient_gpt_amd.plan import AttnPlan
 
+    if args.decode_keys > 0:
+        return decode_bench(args)
     c = CONFIGS[args.cfg]
     if c.dtype != torch.bfloat16 and args.cfg != 1:
         raise SystemExit("unsupported config")

@@ -67,6 +67,12 @@ extern "C" {
                                     QK-norm bound on the logits (sm_scale*D*max|g_q g_k|) would allow the raw
                                     exponent; same results up to rounding, slower */
 
+#define SEGPT_FLAG_DECODE 4      /* forward only, no backward will follow on this kv_workspace: a bf16 call with at most
+                                    32 query rows per kv head (H/Hkv * Sq, the reference's generation step,
+                                    attention.py:191-198) may run the split-key decode kernels, which read k / v /
+                                    v_first once, normalise and rotate on the fly and use kv_workspace for partial
+                                    results instead of normalised keys */
+
 /* which scratch buffer segpt_attn_workspace_bytes() sizes */
 #define SEGPT_WS_KV 0  /* kv_workspace: bf16 copies of the normalised keys (and mixed values); forward AND backward */
 #define SEGPT_WS_BWD 1 /* workspace: per-row statistics, normalised queries, partial sums; backward only            */

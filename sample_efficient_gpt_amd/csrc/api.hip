@@ -179,6 +179,15 @@ size_t segpt_attn_workspace_bytes(const segpt_attn_params* p, int which) {
   return 0;
 }
 
+// A forward-only bf16 call with at most 32 query rows per kv head may take the split-key decode kernels
+// (the caller allows it with SEGPT_FLAG_DECODE; the kv workspace then holds partial results, not keys).
+static bool use_decode(const segpt_attn_params* p) {
+  if (!(p->flags & SEGPT_FLAG_DECODE) || p->dtype != SEGPT_DTYPE_BF16) return false;
+  if ((int64_t)(p->H / p->Hkv) * p->Sq > 32) return false;
+  int kend, splits, chunk;
+  return decode_plan(*p, &kend, &splits, &chunk) <= p->kv_workspace_bytes;
+}
+
 static int fwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi, void* stream) {
   int rc = check_common(p);
   if (rc) return rc;
@@ -187,10 +196,11 @@ static int fwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi
   bind_kv(a);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool f32 = p->dtype == SEGPT_DTYPE_FP32;
+  const bool decode = use_decode(p);
   for (int stage = stage_lo; stage <= stage_hi; ++stage) {
     switch (stage) {
-      case SEGPT_FWD_STAGE_PRE: rc = (f32 || (p->flags & SEGPT_FLAG_KV_PREPARED)) ? 0 : launch_kv_prep(a, st); break;
-      case SEGPT_FWD_STAGE_ATTN: rc = f32 ? launch_fwd_f32(a, st) : launch_fwd_bf16(a, st); break;
+      case SEGPT_FWD_STAGE_PRE: rc = (f32 || decode || (p->flags & SEGPT_FLAG_KV_PREPARED)) ? 0 : launch_kv_prep(a, st); break;
+      case SEGPT_FWD_STAGE_ATTN: rc = f32 ? launch_fwd_f32(a, st) : (decode ? launch_fwd_decode_bf16(a, st) : launch_fwd_bf16(a, st)); break;
       default: return SEGPT_E_STAGE;
     }
     if (rc) return rc;

@@ -24,6 +24,11 @@ struct KArgs {
   float* dcoef_part;  // [n_dkdv_blocks, 2] fp32 partial sums of (dc1, dc2)
   int32_t n_dq_blocks;
   int32_t n_dkdv_blocks;
+  // decode path (split keys): partial O [B*Hkv, splits, 32, D] and (max, sum) [B*Hkv, splits, 32, 2], both fp32,
+  // carved from kv_workspace
+  float* dec_part;
+  float* dec_stat;
+  int32_t dec_splits, dec_chunk, dec_kend;
 };
 
 struct __attribute__((aligned(16))) bf16x8_raw {
@@ -176,6 +181,8 @@ int launch_fwd_bf16(const KArgs& a, hipStream_t st);
 int launch_bwd_dkdv_bf16(const KArgs& a, hipStream_t st);
 int launch_bwd_dq_bf16(const KArgs& a, hipStream_t st);
 int launch_bwd_pre(const KArgs& a, hipStream_t st);     // fp32 path: delta, dgate, do_eff
+int launch_fwd_decode_bf16(KArgs a, hipStream_t st);    // split-key forward for a few query rows against a long cache
+size_t decode_plan(const segpt_attn_params& p, int* kend, int* splits, int* chunk);  // returns its scratch bytes
 int launch_kv_prep(const KArgs& a, hipStream_t st);     // bf16 path: Khat (and V') into kv_workspace
 int launch_bwd_reduce(const KArgs& a, hipStream_t st);  // fp32: dg_q, dg_k, dvr_coef from the partials; bf16: dvr_coef only
 

@@ -88,9 +88,11 @@ def _check_inputs(q, k, v, g_q, g_k, v_first, vr_coef, gate):
         assert gate.shape == (B, Sq, H), "gate_logits must be [B, Sq, H]"
 
 
-def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope=None):
+def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope=None,
+             inference=False):
     """Launch the forward on canonical 4-D views; returns (lse [B,H,Sq] fp32, kv workspace).  `y` is written.
-    The kv workspace holds the normalised keys (and mixed values) the backward can reuse."""
+    The kv workspace holds the normalised keys (and mixed values) the backward can reuse.  `inference`: no
+    backward will follow, so a decode-shaped call (few query rows, long cache) may take the split-key kernels."""
     lib = _lib.load()
     B, H, Sq, _ = q.shape
     lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
@@ -98,6 +100,8 @@ def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scal
     _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope)
     kv_ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_KV, q.device)
     p.kv_workspace, p.kv_workspace_bytes = kv_ws.data_ptr(), kv_ws.numel()
+    if inference:
+        p.flags = _lib.SEGPT_FLAG_DECODE
     rc = lib.segpt_attn_fwd(p, torch.cuda.current_stream(q.device).cuda_stream)
     if rc != 0:
         raise _lib.SegptError(rc, "segpt_attn_fwd")
@@ -151,7 +155,8 @@ class _CoreFunc(torch.autograd.Function):
         y = torch.empty_like(q)
         if y.stride(-1) != 1:
             y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-        lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope)
+        lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope,
+                              inference=not any(ctx.needs_input_grad))
         # the normalised keys (bf16 path) are kept for the backward: 1/rep of q's size
         ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse, kv_ws)
         ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start, rope)
@@ -252,7 +257,7 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
         O = torch.empty_like(Q)
         rope = _rope_arg(rope_cos, rope_sin, None, 0, q_start, Q.device, Q.shape[-1])
         lse, kv_ws = _forward(q4, k4, v4, gq32, gk32, vf4, coef32, gate_logits, gate_scale, eps, sm_scale, is_causal,
-                              q_start, _canon(O, H), rope)
+                              q_start, _canon(O, H), rope, inference=not any(ctx.needs_input_grad))
         ctx.save_for_backward(lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate_logits, kv_ws)
         ctx.cfg = (H, Hkv, gate_scale, eps, sm_scale, bool(is_causal), int(q_start), rope)
         return O

@@ -289,6 +289,40 @@ def test_fused_rope_equals_rotating_first_and_rejects_bad_tables(gpu_device):
         run_gpu(xf, gpu_device, backward=False, rope=(cos, sin))
 
 
+# ------------------------------------------------------------------ decode-shaped calls (split-key kernels)
+
+
+@pytest.mark.parametrize(
+    "B,H,Hkv,Sq,Sk,D,kw,gen_kw,use_rope",
+    [
+        (1, 18, 6, 1, 2048, 64, {"q_start": 2047}, {}, False),          # one new token against a 2048-key cache
+        (2, 6, 2, 1, 1000, 64, {"q_start": 999}, {}, True),             # ragged cache length, rotary positions
+        (1, 6, 2, 4, 777, 64, {"q_start": 773}, {"extras": True}, True),  # 4 new tokens, gate + value residual
+        (1, 8, 1, 3, 300, 64, {"q_start": 297}, {"scalar_gain": True, "no_gk": True}, False),  # 24 rows per kv head
+        (3, 4, 4, 1, 129, 128, {"q_start": 128}, {}, True),
+        (1, 4, 2, 2, 640, 128, {"causal": False}, {}, False),
+        (16, 6, 2, 1, 4096, 64, {"q_start": 4095}, {}, False),          # many groups: few splits each
+    ],
+)
+def test_decode_path_matches_oracle_and_training_kernel(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw, use_rope):
+    """Forward-only calls with H/Hkv * Sq <= 32 take the split-key decode kernels (through the C ABI, flag
+    SEGPT_FLAG_DECODE set by the front end when nothing requires grad); same tolerance against the oracle, and
+    agreement with the training kernel on the same inputs."""
+    x = gen(B, H, Hkv, Sq, Sk, D, BF16, seed=41, **gen_kw)
+    if use_rope:
+        kw = dict(kw, rope=orc.rope_tables(Sk + 8, 10000.0, D))
+    print(f"decode case B={B} H={H} Hkv={Hkv} Sq={Sq} Sk={Sk} D={D} kw={ {k: v for k, v in kw.items() if k != 'rope'} } rope={use_rope}", flush=True)
+    ref = run_oracle(x, backward=False, **kw)
+    with torch.no_grad():
+        dec = run_gpu(x, gpu_device, backward=False, **kw)          # inference: decode kernels
+    compare(dec, ref, BF16)
+    xg = dict(x)
+    trn = run_gpu(xg, gpu_device, backward=True, **kw)                # needs grad: training kernels
+    compare({n: trn[n] for n in ("y", "lse")}, ref, BF16)
+    assert torch.allclose(dec["y"].float(), trn["y"].float(), atol=2e-2, rtol=1e-2)
+    assert torch.allclose(dec["lse"], trn["lse"], atol=2e-2, rtol=1e-2)
+
+
 def test_backward_is_deterministic(gpu_device):
     x = gen(2, 6, 2, 512, 512, 64, BF16, extras=True, seed=4)
     a = run_gpu(x, gpu_device)
