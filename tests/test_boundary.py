@@ -41,6 +41,11 @@ def test_header_constants_match_binding():
     assert int(consts["SEGPT_ABI_VERSION"]) == _lib.SEGPT_ABI_VERSION
     assert int(consts["SEGPT_DTYPE_BF16"]) == _lib.SEGPT_DTYPE_BF16
     assert int(consts["SEGPT_DTYPE_FP32"]) == _lib.SEGPT_DTYPE_FP32
+    for name in ("SEGPT_FLAG_KV_PREPARED", "SEGPT_FLAG_RUNNING_MAX", "SEGPT_FLAG_DECODE", "SEGPT_WS_KV", "SEGPT_WS_BWD"):
+        assert int(consts[name]) == getattr(_lib, name), name
+    stages = lambda prefix: [k for k, _ in sorted(((k, int(v)) for k, v in consts.items() if k.startswith(prefix)), key=lambda kv: kv[1])]
+    assert [s.rsplit("_", 1)[1].lower() for s in stages("SEGPT_FWD_STAGE_")] == list(_lib.FWD_STAGES)
+    assert [s.rsplit("_", 1)[1].lower() for s in stages("SEGPT_BWD_STAGE_")] == list(_lib.BWD_STAGES)
     # every error code has its own text
     texts = {_lib.strerror(int(v)) for k, v in consts.items() if k.startswith("SEGPT_E_")}
     assert len(texts) == len([k for k in consts if k.startswith("SEGPT_E_")])
@@ -102,6 +107,17 @@ def test_argument_errors_are_reported_before_any_launch(lib):
     assert lib.segpt_attn_fwd(p, None) == -10
     assert lib.segpt_attn_fwd_stage(_valid_params(), 2, None) == -11
     assert lib.segpt_attn_bwd_stage(_valid_params(), 4, None) == -11
+    # rotary tables: both or neither, aligned, long enough for the positions, bf16 only
+    p = _valid_params(); p.rope_cos = 0x50000
+    assert lib.segpt_attn_fwd(p, None) == -12
+    p = _valid_params(); p.rope_cos, p.rope_sin, p.rope_len = 0x50000, 0x60000, 127  # Sq = Sk = 128 rows
+    assert lib.segpt_attn_fwd(p, None) == -12
+    p.rope_len, p.rope_q_pos0 = 128, 1
+    assert lib.segpt_attn_fwd(p, None) == -12
+    p.rope_q_pos0, p.rope_sin = 0, 0x60004
+    assert lib.segpt_attn_fwd(p, None) == -12
+    p = _valid_params(dtype=_lib.SEGPT_DTYPE_FP32); p.rope_cos, p.rope_sin, p.rope_len = 0x50000, 0x60000, 4096
+    assert lib.segpt_attn_fwd(p, None) == -12
     # backward-only checks
     p = _valid_params()
     assert lib.segpt_attn_bwd(p, None) == -7  # no workspace
