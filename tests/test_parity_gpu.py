@@ -302,6 +302,10 @@ def test_fused_rope_equals_rotating_first_and_rejects_bad_tables(gpu_device):
         (3, 4, 4, 1, 129, 128, {"q_start": 128}, {}, True),
         (1, 4, 2, 2, 640, 128, {"causal": False}, {}, False),
         (16, 6, 2, 1, 4096, 64, {"q_start": 4095}, {}, False),          # many groups: few splits each
+        (1, 32, 1, 1, 513, 64, {"q_start": 512}, {}, False),            # exactly 32 query rows per kv head
+        (2, 4, 2, 2, 500, 64, {"q_start": 10}, {}, True),               # only the first 12 keys are visible
+        (1, 4, 2, 1, 5, 64, {"q_start": 4}, {}, False),                 # cache shorter than one key block
+        (1, 2, 2, 1, 1, 64, {"q_start": 0}, {}, True),                  # the very first token: one key
     ],
 )
 def test_decode_path_matches_oracle_and_training_kernel(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw, use_rope):
