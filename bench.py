@@ -192,6 +192,7 @@ def main():
     torch.cuda.synchronize()
     ms_staged = (time.perf_counter() - t1) / args.steps * 1e3
     kern_ms = {n: sum(e[j].elapsed_time(e[j + 1]) for e in evs) / args.steps for j, n in enumerate(names)}
+    step_ms = sorted(e[0].elapsed_time(e[len(names)]) for e in evs)  # first to last event of each replayed step
 
     unit = c.B * c.H * c.S * c.S * c.D  # one causal S x S x D contraction, in FLOPs
     credited = {"fwd": 2 * unit, "bwd_dkdv": 4 * unit, "bwd_dq": 1 * unit}  # dq's recomputed S and dP are not credited
@@ -235,6 +236,8 @@ def main():
         },
         "pct_of_bf16_mfma_peak": round(100 * value / MI355X_BF16_DENSE_TFLOPS, 2),
         "ms_per_step_with_stage_events": round(ms_staged, 5),
+        "staged_step_ms_median": round(step_ms[len(step_ms) // 2], 5),
+        "staged_step_ms_min": round(step_ms[0], 5),
         "roofline": {
             "kernel": dom,
             "bound": "mfma",
