@@ -73,6 +73,12 @@ extern "C" {
                                     v_first once, normalise and rotate on the fly and use kv_workspace for partial
                                     results instead of normalised keys */
 
+#define SEGPT_FLAG_NO_NORM 8     /* plain attention: both RMS normalisers are exactly 1 (eps is ignored), so
+                                    s_ij = sm_scale * (q_i o g_q) . (k_j o g_k); with g_q = 1 and no g_k this is the
+                                    reference's non-QK-norm path, TritonFlashAttnFunc (triton_flash_attn.py:208-297)
+                                    and the SDPA call attention.py:233-240.  Logits are then unbounded: the bf16
+                                    forward always keeps a running row maximum */
+
 /* which scratch buffer segpt_attn_workspace_bytes() sizes */
 #define SEGPT_WS_KV 0  /* kv_workspace: bf16 copies of the normalised keys (and mixed values); forward AND backward */
 #define SEGPT_WS_BWD 1 /* workspace: per-row statistics, normalised queries, partial sums; backward only            */

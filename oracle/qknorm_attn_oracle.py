@@ -12,6 +12,9 @@ reference computes on its attention path:
   (L2 normaliser, eps 1e-8 on the sum, logit = gain*cos)  -> ``fused_kernel_variant_b``
 * the CPU monkey patch `sample_efficient_gpt/scripts/hf/convert_imu1_checkpoint.py:73-89`
   (RMS, eps 1e-8, logit = gain*d*cos)                     -> ``cpu_patch_variant_c``
+* the attention without QK-norm, `attention.py:233-240` (SDPA) and `TritonFlashAttnFunc`,
+  `sample_efficient_gpt/transformer/ops/triton_flash_attn.py:208-297`   -> ``plain_flash_variant``
+  (the family with ``qk_norm=False``)
 * the caller glue of `attention.py:199-255`: `(h b)` head-major flatten, GQA
   `repeat_interleave`, value-residual mix, per-head `2*sigmoid` gate
                                                           -> ``flatten_heads`` ... ``caller_glue``
@@ -31,6 +34,8 @@ this path, so every pin is mathematical -- see tests/test_oracle.py):
   ``torch.autograd`` through ``attention_forward`` in fp64 and ``gradcheck``.
 * variants A/B/C           each written from its own reference lines with its own
   normaliser; pinned by the family remap (eps, sm_scale) equality in fp64.
+* ``plain_flash_variant``   pinned against ``F.scaled_dot_product_attention`` and the family with
+  ``qk_norm=False``; the ``qk_norm=False`` explicit backward against autograd in fp64.
 * layout helpers           pinned by brute-force python indexing on tiny tensors.
 
 The exact bf16 rounding order of variant A (normalise -> round -> times
@@ -119,6 +124,7 @@ def attention_forward(
     rope=None,
     rope_q_pos0: int | None = None,
     rope_k_pos0: int = 0,
+    qk_norm: bool = True,
 ):
     """Generalised QK-norm attention in canonical layout.
 
@@ -128,6 +134,8 @@ def attention_forward(
     rope = (cos, sin) tables: q and k are rotated before the normalisation, as the reference's caller does
     (attention.py:202-204); query row i sits at position rope_q_pos0 + i (default q_start, attention.py:191-195),
     key row j at rope_k_pos0 + j.
+    qk_norm=False: both normalisers are 1 (eps unused) -- the reference's attention without QK-norm
+    (attention.py:233-240, triton_flash_attn.py:208-297) when g_q = 1 and g_k is None.
     Computes in the dtype of ``q`` (callers pass fp32 or fp64).
     Returns (y, lse, o_ungated, v_mixed); lse is in natural-log units.
     """
@@ -143,8 +151,8 @@ def attention_forward(
         q = apply_rope(q, rope[0], rope[1], q_start if rope_q_pos0 is None else rope_q_pos0)
         k = apply_rope(k, rope[0], rope[1], rope_k_pos0)
 
-    qn = q * rms_inv(q, eps) * gq
-    kn = k * rms_inv(k, eps) * gk
+    qn = q * (rms_inv(q, eps) if qk_norm else 1.0) * gq
+    kn = k * (rms_inv(k, eps) if qk_norm else 1.0) * gk
     if vr_coef is not None:
         assert v_first is not None
         c = vr_coef if torch.is_tensor(vr_coef) else torch.tensor(vr_coef, dtype=q.dtype)
@@ -205,6 +213,7 @@ def attention_backward_explicit(
     vr_coef=None,
     gate_logits=None,
     gate_scale=2.0,
+    qk_norm=True,
 ):
     """Hand-written chain rule (no autograd).  Returns a dict of gradients.
 
@@ -222,7 +231,7 @@ def attention_backward_explicit(
     gk = _vec(g_k, D, q)
     y, lse, o, vm = attention_forward(
         q, k, v, g_q, g_k, eps=eps, sm_scale=sm_scale, causal=causal, q_start=q_start,
-        v_first=v_first, vr_coef=vr_coef, gate_logits=gate_logits, gate_scale=gate_scale,
+        v_first=v_first, vr_coef=vr_coef, gate_logits=gate_logits, gate_scale=gate_scale, qk_norm=qk_norm,
     )
     out = {}
     # gate
@@ -235,8 +244,9 @@ def attention_backward_explicit(
         do = dy
     delta = (do * o).sum(-1)  # [B,H,Sq]
 
-    a = rms_inv(q, eps)  # [B,H,Sq,1]
-    b = rms_inv(k, eps)
+    a = rms_inv(q, eps) if qk_norm else torch.ones_like(q[..., :1])  # [B,H,Sq,1]
+    b = rms_inv(k, eps) if qk_norm else torch.ones_like(k[..., :1])
+    proj = 1.0 if qk_norm else 0.0  # without a normaliser its own gradient term vanishes
     qn = q * a * gq
     kn = k * b * gk
     kx = kn.repeat_interleave(rep, dim=1)
@@ -256,10 +266,10 @@ def attention_backward_explicit(
 
     # through the normalisers:  x~ = a x * g,  a = rsqrt(mean x^2 + eps)
     u = dqn * gq
-    out["dq"] = a * u - (a**3 / D) * (u * q).sum(-1, keepdim=True) * q
+    out["dq"] = a * u - proj * (a**3 / D) * (u * q).sum(-1, keepdim=True) * q
     out["dg_q"] = (dqn * (a * q)).sum(dim=(0, 1, 2))
     w = dkn * gk
-    out["dk"] = b * w - (b**3 / D) * (w * k).sum(-1, keepdim=True) * k
+    out["dk"] = b * w - proj * (b**3 / D) * (w * k).sum(-1, keepdim=True) * k
     out["dg_k"] = (dkn * (b * k)).sum(dim=(0, 1, 2))
 
     if vr_coef is not None:
@@ -365,6 +375,20 @@ def cpu_patch_variant_c(Q, K, V, gain, is_causal: bool = True, q_start: int = 0)
 
 
 # --------------------------------------------------------------------------- caller glue (attention.py:199-255)
+
+
+def plain_flash_variant(Q, K, V, q_start: int = 0, is_causal: bool = True):
+    """The reference's attention WITHOUT QK-norm on flattened [(h b), S, d] tensors: softmax(Q K^T / sqrt(d)) V
+    with the `k_idx <= q_start + q_idx` mask -- TritonFlashAttnFunc (triton_flash_attn.py:208-297, scale at
+    :232; note the argument order q_start, is_causal) and the SDPA call attention.py:233-236.  Written as
+    the brute-force softmax; the family reaches it with qk_norm=False, g_q = 1.  The reference kernel's
+    backward mis-masks one diagonal tile when BQ != BK (triton_flash_attn.py:176,292-293); this restatement
+    is the exact mathematics instead."""
+    d = Q.shape[-1]
+    s = torch.einsum("nid,njd->nij", Q, K) / math.sqrt(d)
+    vis = visibility_mask(Q.shape[1], K.shape[1], is_causal, q_start, device=Q.device)
+    s = s.masked_fill(~vis, float("-inf"))
+    return torch.einsum("nij,njd->nid", torch.softmax(s, dim=-1), V)
 
 
 def flatten_heads(x):

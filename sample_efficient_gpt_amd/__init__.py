@@ -7,10 +7,11 @@ canonical ``[B, H, S, D]`` views.  All compute runs in hand-written HIP kernels 
 through the C ABI of ``libsegpt_attn.so``; there is no fallback path.
 """
 
-from .function import QKNormFlashAttnFunc, qknorm_attention  # noqa: F401
+from .function import FlashAttnFunc, QKNormFlashAttnFunc, qknorm_attention  # noqa: F401
 from .module import SelfDotProductAttnQKNorm  # noqa: F401
 from .library_op import qknorm_attention_op  # noqa: F401  (registers torch.ops.segpt.qknorm_attention)
 from .inputs import CONFIGS, AttnConfig, make_inputs  # noqa: F401
 
 # the reference's class name, so `from ... import TritonFlashAttnQKNormFunc` call sites keep working
 TritonFlashAttnQKNormFunc = QKNormFlashAttnFunc
+TritonFlashAttnFunc = FlashAttnFunc

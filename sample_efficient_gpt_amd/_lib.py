@@ -18,6 +18,7 @@ SEGPT_DTYPE_FP32 = 1
 SEGPT_FLAG_KV_PREPARED = 1
 SEGPT_FLAG_RUNNING_MAX = 2
 SEGPT_FLAG_DECODE = 4
+SEGPT_FLAG_NO_NORM = 8
 SEGPT_WS_KV = 0
 SEGPT_WS_BWD = 1
 FWD_STAGES = ("pre", "attn")  # SEGPT_FWD_STAGE_* = index

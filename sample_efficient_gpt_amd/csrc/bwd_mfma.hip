@@ -122,7 +122,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
       for (int t = 0; t < 8; ++t) ss += qx[ks][t] * qx[ks][t];
     ss = half_sum(ss);
     delta = half_sum(dl);
-    alpha = fast_rsq(ss * (1.0f / D) + p.eps);
+    alpha = row_normaliser_fast(p, ss, 1.0f / D);
     const float f = alpha * p.sm_scale * kLog2e;
     float gfac = 1.f;
     if (p.gate.ptr) {
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     }
   }
   dot = half_sum(dot);
-  const float a3 = alpha * alpha * alpha * (1.0f / D) * dot;
+  const float a3 = norm_grad_coef(p, alpha, 1.0f / D) * dot;
   uint16_t* op = row_ptr_mut<uint16_t>(p.dq, b, h, row_c);
   float val[MB][16];
 #pragma unroll
@@ -549,8 +549,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
       for (int r = 0; r < 16; ++r) { dot += dkacc[mb][r] * kv[mb][r]; ss += kv[mb][r] * kv[mb][r]; }
     dot = half_sum(dot) * kLn2;
     ss = half_sum(ss);
-    const float beta = fast_rsq(ss * (1.0f / D) + p.eps);
-    const float b3 = beta * beta * beta * (1.0f / D) * dot;
+    const float beta = row_normaliser_fast(p, ss, 1.0f / D);
+    const float b3 = norm_grad_coef(p, beta, 1.0f / D) * dot;
     uint16_t* okp = row_ptr_mut<uint16_t>(p.dk, b, g, key_c);
     float val[MB][16];
 #pragma unroll

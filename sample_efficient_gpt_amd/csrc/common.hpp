@@ -31,6 +31,19 @@ struct KArgs {
   int32_t dec_splits, dec_chunk, dec_kend;
 };
 
+// Row normaliser 1/sqrt(mean x^2 + eps) from the row's sum of squares ss (inv_d = 1/D); exactly 1 for plain
+// attention (SEGPT_FLAG_NO_NORM).
+__device__ __forceinline__ float row_normaliser(const segpt_attn_params& p, float ss, float inv_d) {
+  return (p.flags & SEGPT_FLAG_NO_NORM) ? 1.0f : 1.0f / sqrtf(ss * inv_d + p.eps);
+}
+__device__ __forceinline__ float row_normaliser_fast(const segpt_attn_params& p, float ss, float inv_d) {
+  return (p.flags & SEGPT_FLAG_NO_NORM) ? 1.0f : __builtin_amdgcn_rsqf(ss * inv_d + p.eps);
+}
+// n^3/D, the factor of the normaliser's own term in dx = n u - (n^3/D)(u.x) x; 0 when there is no normaliser
+__device__ __forceinline__ float norm_grad_coef(const segpt_attn_params& p, float n, float inv_d) {
+  return (p.flags & SEGPT_FLAG_NO_NORM) ? 0.0f : n * n * n * inv_d;
+}
+
 struct __attribute__((aligned(16))) bf16x8_raw {
   uint32_t w[4];
 };

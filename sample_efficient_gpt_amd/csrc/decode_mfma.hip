@@ -86,7 +86,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(KArgs a) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) ss += x[ks][t] * x[ks][t];
     ss = half_sum(ss);
-    const float alpha = qlive ? fast_rsq(ss * (1.0f / D) + p.eps) : 0.f;
+    const float alpha = qlive ? row_normaliser_fast(p, ss, 1.0f / D) : 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const float4 ga = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh);
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(KArgs a) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) ss += kx[ks][t] * kx[ks][t];
     ss = half_sum(ss);
-    const float beta = fast_rsq(ss * (1.0f / D) + p.eps);
+    const float beta = row_normaliser_fast(p, ss, 1.0f / D);
     f32x16 s = splat16(0.f);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {

@@ -72,7 +72,7 @@ __device__ __forceinline__ void stage_kv(const segpt_attn_params& p, int b, int 
 #pragma unroll
   for (int e = 0; e < PT; ++e) ss += kreg[e] * kreg[e];
   ss = oct_sum(ss);
-  const float beta = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
+  const float beta = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
   for (int e = 0; e < PT; ++e) {
     kh[r * D + part * PT + e] = kreg[e] * beta;
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void fwd_f32_kernel(KArgs a) {
       for (int x = 0; x < 4; ++x) { qh[e + x] = t[x]; ss += t[x] * t[x]; }
     }
     ss = quad_sum(ss);
-    const float alpha = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
+    const float alpha = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
     for (int e = 0; e < DP; ++e) {
       qh[e] = qh[e] * alpha * gprod<D>(p, sub * DP + e) * p.sm_scale;
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_f32_kernel(KArgs a) {
       for (int x = 0; x < 4; ++x) dout[e + x] = t[x];
     }
     ss = quad_sum(ss);
-    alpha = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
+    alpha = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
     for (int e = 0; e < DP; ++e) {
       qh[e] = qraw[e] * alpha * gprod<D>(p, sub * DP + e) * p.sm_scale;
@@ -250,7 +250,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_f32_kernel(KArgs a) {
   }
   dot = quad_sum(dot);
   if (live) {
-    const float a3 = alpha * alpha * alpha * (1.0f / D) * dot;
+    const float a3 = norm_grad_coef(p, alpha, 1.0f / D) * dot;
     float* op = row_ptr_mut<float>(p.dq, b, h, row) + sub * DP;
 #pragma unroll
     for (int e = 0; e < DP; e += 4) {
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkdv_f32_kernel(KArgs a) {
       }
     }
     ss = quad_sum(ss);
-    beta = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
+    beta = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
     for (int e = 0; e < DP; ++e) {
       kh[e] *= beta;
@@ -365,7 +365,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkdv_f32_kernel(KArgs a) {
 #pragma unroll
         for (int e = 0; e < PT; ++e) ss += qreg[e] * qreg[e];
         ss = oct_sum(ss);
-        const float alpha = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
+        const float alpha = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
         for (int e = 0; e < PT; ++e) {
           qs[r * D + part * PT + e] = qreg[e] * alpha * gprod<D>(p, part * PT + e) * p.sm_scale;
@@ -411,7 +411,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkdv_f32_kernel(KArgs a) {
   }
   dot = quad_sum(dot);
   if (live) {
-    const float b3 = beta * beta * beta * (1.0f / D) * dot;
+    const float b3 = norm_grad_coef(p, beta, 1.0f / D) * dot;
     float* okp = row_ptr_mut<float>(p.dk, b, g, j) + sub * DP;
     float* ovp = row_ptr_mut<float>(p.dv, b, g, j) + sub * DP;
 #pragma unroll

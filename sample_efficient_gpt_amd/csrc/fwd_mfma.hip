@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
   const int b = wg.b, g = wg.g, h = wg.g * rep + wg.hh;
   const int q0 = wg.tile * BQ;
   const int qw0 = q0 + wave * 32 * NQB;  // first query of this wave
-  const bool bounded = !(p.flags & SEGPT_FLAG_RUNNING_MAX) && logit_bound(p, lane) <= kNoMaxBound;  // wave-uniform
+  const bool bounded = !(p.flags & (SEGPT_FLAG_RUNNING_MAX | SEGPT_FLAG_NO_NORM)) && logit_bound(p, lane) <= kNoMaxBound;  // wave-uniform
 
   int kend = p.Sk;
   if (p.causal) kend = min(p.Sk, q0 + BQ + p.q_start);
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
 #pragma unroll
       for (int t = 0; t < 8; ++t) ss += x[ks][t] * x[ks][t];
     ss = half_sum(ss);
-    const float alpha = fast_rsq(ss * (1.0f / D) + p.eps);
+    const float alpha = row_normaliser_fast(p, ss, 1.0f / D);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const float4 ga = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh);

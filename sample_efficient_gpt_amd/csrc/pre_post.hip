@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void bwd_pre_kernel(KArgs a) {
     }
     if (!live) continue;
     if (a.qhat) {  // bf16 path: the normalised, scaled query row the two MFMA kernels consume
-      const float f = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
+      const float f = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
       for (int e = 0; e < V; ++e) q[e] *= f * gs[e];
       Elem<T>::store(reinterpret_cast<T*>(a.qhat) + r * D + part * V, q);
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void kv_prep_kernel(KArgs a) {
   for (int e = 0; e < 8; ++e) ss += k[e] * k[e];
 #pragma unroll
   for (int o = 1; o < TPR; o <<= 1) ss += __shfl_xor(ss, o, 64);
-  const float beta = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
+  const float beta = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
   for (int e = 0; e < 8; ++e) k[e] *= beta;
   if (live) Elem<uint16_t>::store(a.khat + r * D + part * 8, k);

@@ -89,10 +89,11 @@ def _check_inputs(q, k, v, g_q, g_k, v_first, vr_coef, gate):
 
 
 def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope=None,
-             inference=False):
+             inference=False, flags=0):
     """Launch the forward on canonical 4-D views; returns (lse [B,H,Sq] fp32, kv workspace).  `y` is written.
     The kv workspace holds the normalised keys (and mixed values) the backward can reuse.  `inference`: no
-    backward will follow, so a decode-shaped call (few query rows, long cache) may take the split-key kernels."""
+    backward will follow, so a decode-shaped call (few query rows, long cache) may take the split-key kernels.
+    `flags`: SEGPT_FLAG_* bits of the call itself (SEGPT_FLAG_NO_NORM for attention without QK-norm)."""
     lib = _lib.load()
     B, H, Sq, _ = q.shape
     lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
@@ -100,8 +101,7 @@ def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scal
     _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope)
     kv_ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_KV, q.device)
     p.kv_workspace, p.kv_workspace_bytes = kv_ws.data_ptr(), kv_ws.numel()
-    if inference:
-        p.flags = _lib.SEGPT_FLAG_DECODE
+    p.flags = flags | (_lib.SEGPT_FLAG_DECODE if inference else 0)
     rc = lib.segpt_attn_fwd(p, torch.cuda.current_stream(q.device).cuda_stream)
     if rc != 0:
         raise _lib.SegptError(rc, "segpt_attn_fwd")
@@ -109,7 +109,7 @@ def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scal
 
 
 def _backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, y, lse, dy,
-              dq, dk, dv, dv_first, dgate, kv_ws=None, rope=None):
+              dq, dk, dv, dv_first, dgate, kv_ws=None, rope=None, flags=0):
     """Launch the backward; dq/dk/dv(/dv_first/dgate) are written; returns (dg_q, dg_k, dvr_coef) fp32.
     `kv_ws`: the forward's kv workspace (skips the key/value pre-pass); None allocates a fresh one."""
     lib = _lib.load()
@@ -125,10 +125,11 @@ def _backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_sca
     p.dg_q, p.dg_k, p.dvr_coef = _lib.ptr(dg_q), _lib.ptr(dg_k), _lib.ptr(dcoef)
     ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_BWD, dev)
     p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    p.flags = flags
     if kv_ws is None:
         kv_ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_KV, dev)
     else:
-        p.flags = _lib.SEGPT_FLAG_KV_PREPARED
+        p.flags |= _lib.SEGPT_FLAG_KV_PREPARED
     p.kv_workspace, p.kv_workspace_bytes = kv_ws.data_ptr(), kv_ws.numel()
     rc = lib.segpt_attn_bwd(p, torch.cuda.current_stream(dev).cuda_stream)
     if rc != 0:
@@ -144,7 +145,8 @@ class _CoreFunc(torch.autograd.Function):
     """Canonical-layout op: q [B,H,Sq,D], k/v/v_first [B,Hkv,Sk,D], gate [B,Sq,H]."""
 
     @staticmethod
-    def forward(ctx, q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope=None):
+    def forward(ctx, q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope=None,
+                flags=0):
         gq32, gk32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device)
         coef32 = None if vr_coef is None else vr_coef.detach().to(device=q.device, dtype=torch.float32).reshape(-1).contiguous()
         _check_inputs(q, k, v, gq32, gk32, v_first, coef32, gate)
@@ -156,17 +158,17 @@ class _CoreFunc(torch.autograd.Function):
         if y.stride(-1) != 1:
             y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope,
-                              inference=not any(ctx.needs_input_grad))
+                              inference=not any(ctx.needs_input_grad), flags=flags)
         # the normalised keys (bf16 path) are kept for the backward: 1/rep of q's size
         ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse, kv_ws)
-        ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start, rope)
+        ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start, rope, flags)
         ctx.mark_non_differentiable(lse)
         return y, lse
 
     @staticmethod
     def backward(ctx, dy, _dlse):
         q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse, kv_ws = ctx.saved_tensors
-        gate_scale, eps, sm_scale, causal, q_start, rope = ctx.cfg
+        gate_scale, eps, sm_scale, causal, q_start, rope, flags = ctx.cfg
         gq32, gk32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device)
         coef32 = None if vr_coef is None else vr_coef.detach().to(device=q.device, dtype=torch.float32).reshape(-1).contiguous()
         dy = _lastdim_contig(dy)
@@ -176,18 +178,18 @@ class _CoreFunc(torch.autograd.Function):
         dv_first = None if v_first is None else torch.empty_like(v_first)
         dgate = None if gate is None else torch.empty_like(gate)
         dg_q, dg_k, dcoef = _backward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal,
-                                      q_start, y, lse, dy, dq, dk, dv, dv_first, dgate, kv_ws, rope)
+                                      q_start, y, lse, dy, dq, dk, dv, dv_first, dgate, kv_ws, rope, flags)
         dg_q = dg_q.reshape(g_q.shape).to(g_q.dtype)
         if g_k is not None:
             dg_k = dg_k.reshape(g_k.shape).to(g_k.dtype)
         if vr_coef is not None:
             dcoef = dcoef.reshape(vr_coef.shape).to(vr_coef.dtype)
-        return dq, dk, dv, dg_q, dg_k, dv_first, dcoef, dgate, None, None, None, None, None, None
+        return dq, dk, dv, dg_q, dg_k, dv_first, dcoef, dgate, None, None, None, None, None, None, None
 
 
 def qknorm_attention(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate_logits=None, gate_scale=2.0,
                      eps=1e-6, sm_scale=None, causal=True, q_start=0, return_lse=False,
-                     rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0):
+                     rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0, qk_norm=True):
     """Fused QK-norm attention on canonical views.
 
     q ``[B,H,Sq,D]``; k, v, v_first ``[B,Hkv,Sk,D]`` (any strides, last dim contiguous, rows 16 B
@@ -196,10 +198,12 @@ def qknorm_attention(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate
     rope_cos / rope_sin ``[len, D/2]``: q and k are the UNROTATED projections and the split-half rotary
     embedding (rope.py:36-56) is applied inside the kernels' loads (bf16 only); query row i sits at position
     ``rope_q_pos0 + i`` (default ``q_start``), key row j at ``rope_k_pos0 + j``.
+    ``qk_norm=False``: no RMS normalisation of q and k (eps unused) -- the reference's attention without QK-norm
+    (attention.py:233-240); the scale vectors still apply, pass ``g_q = ones(1)`` for the plain op.
     """
     rope = _rope_arg(rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, q_start, q.device, q.shape[-1])
     y, lse = _CoreFunc.apply(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
-                             rope)
+                             rope, 0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM)
     return (y, lse) if return_lse else y
 
 
@@ -286,3 +290,54 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
         dcoef = None if vr_coef is None else dcoef.reshape(vr_coef.shape).to(vr_coef.dtype)
         #      Q   K   V   gain   causal q_start k_gain  v_first vr_coef gate  gate_scale n_kv eps sm_scale rope tables
         return dQ, dK, dV, dgain, None, None, dk_gain, dVf, dcoef, dgate, None, None, None, None, None, None
+
+
+class FlashAttnFunc(torch.autograd.Function):
+    """Drop-in for the reference's attention WITHOUT QK-norm, ``TritonFlashAttnFunc``
+    (triton_flash_attn.py:208-297; called at attention.py:240): ``apply(Q, K, V, q_start=0, is_causal=True,
+    n_kv_heads=None)`` -- note the argument order, which differs from the QK-norm op's.  ``Q [(h b), Nq, d]``,
+    ``K, V [(h b) or (hkv b), Nk, d]`` contiguous device tensors (2-D promoted to 3-D, :222-226); logits are
+    ``Q K^T / sqrt(d)`` (:232).  Same kernels as the QK-norm op with both normalisers fixed at 1
+    (SEGPT_FLAG_NO_NORM).  The reference backward's mis-masked diagonal tile (BQ=32 != BK=64,
+    triton_flash_attn.py:176,292-293) is not reproduced: gradients are the exact ones."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, q_start=0, is_causal=True, n_kv_heads=None):
+        assert Q.is_cuda and Q.is_contiguous()
+        assert K.is_cuda and K.is_contiguous()
+        assert V.is_cuda and V.is_contiguous()
+        if Q.ndim == 2:
+            Q, K, V = Q.unsqueeze(0), K.unsqueeze(0), V.unsqueeze(0)
+        nq, nk = Q.shape[0], K.shape[0]
+        if n_kv_heads is None:
+            assert nk == nq, "n_kv_heads is required for un-expanded GQA K/V"
+            H = Hkv = 1
+        else:
+            Hkv = int(n_kv_heads)
+            assert nq % nk == 0 and nk % Hkv == 0, "K/V rows must be n_kv_heads * batch"
+            H = Hkv * (nq // nk)
+        q4, k4, v4 = _canon(Q, H), _canon(K, Hkv), _canon(V, Hkv)
+        one = torch.ones(1, dtype=torch.float32, device=Q.device)
+        _check_inputs(q4, k4, v4, one, None, None, None, None)
+        sm_scale = 1.0 / math.sqrt(Q.shape[-1])
+        O = torch.empty_like(Q)
+        lse, kv_ws = _forward(q4, k4, v4, one, None, None, None, None, 1.0, 0.0, sm_scale, is_causal, q_start, _canon(O, H),
+                              None, inference=not any(ctx.needs_input_grad), flags=_lib.SEGPT_FLAG_NO_NORM)
+        ctx.save_for_backward(lse, Q, K, V, O, one, kv_ws)
+        ctx.cfg = (H, Hkv, sm_scale, bool(is_causal), int(q_start))
+        return O
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        lse, Q, K, V, O, one, kv_ws = ctx.saved_tensors
+        H, Hkv, sm_scale, causal, q_start = ctx.cfg
+        grad_output = grad_output.contiguous()
+        if grad_output.dtype != Q.dtype:
+            grad_output = grad_output.to(Q.dtype)
+        if grad_output.ndim == 2:
+            grad_output = grad_output.unsqueeze(0)
+        dQ, dK, dV = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+        _backward(_canon(Q, H), _canon(K, Hkv), _canon(V, Hkv), one, None, None, None, None, 1.0, 0.0, sm_scale, causal,
+                  q_start, _canon(O, H), lse, _canon(grad_output, H), _canon(dQ, H), _canon(dK, Hkv), _canon(dV, Hkv),
+                  None, None, kv_ws, None, _lib.SEGPT_FLAG_NO_NORM)
+        return dQ, dK, dV, None, None, None

@@ -5,7 +5,7 @@ non-reentrant activation checkpointing (transformer/transformer.py:123-132) as O
 
     y = torch.ops.segpt.qknorm_attention(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits,
                                          gate_scale, eps, sm_scale, causal, q_start,
-                                         rope_cos, rope_sin, rope_q_pos0, rope_k_pos0)[0]
+                                         rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm)[0]
 
 or the keyword wrapper ``qknorm_attention_op(...)`` below.  Canonical layout: q ``[B,H,Sq,D]``, k / v /
 v_first ``[B,Hkv,Sk,D]`` (any strides, last dim contiguous), gate_logits ``[B,Sq,H]``; the optional tensors
@@ -35,20 +35,21 @@ def _coef32(vr_coef, device):
 def _fwd_op(q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optional[Tensor], v_first: Optional[Tensor],
             vr_coef: Optional[Tensor], gate_logits: Optional[Tensor], gate_scale: float, eps: float, sm_scale: float,
             causal: bool, q_start: int, rope_cos: Optional[Tensor], rope_sin: Optional[Tensor],
-            rope_q_pos0: int, rope_k_pos0: int) -> List[Tensor]:
+            rope_q_pos0: int, rope_k_pos0: int, qk_norm: bool) -> List[Tensor]:
     rope = _rope_arg(rope_cos, rope_sin, None if rope_q_pos0 < 0 else rope_q_pos0, rope_k_pos0, q_start, q.device, q.shape[-1])
     gq32, gk32, c32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device), _coef32(vr_coef, q.device)
     _check_inputs(q, k, v, gq32, gk32, v_first, c32, gate_logits)
     q, k, v = _lastdim_contig(q), _lastdim_contig(k), _lastdim_contig(v)
     v_first = None if v_first is None else _lastdim_contig(v_first)
     y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, c32, gate_logits, gate_scale, eps, sm_scale, causal, q_start, y, rope)
+    lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, c32, gate_logits, gate_scale, eps, sm_scale, causal, q_start, y, rope,
+                          flags=0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM)
     return [y, lse, kv_ws]
 
 
 @_fwd_op.register_fake
 def _(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
-      rope_cos, rope_sin, rope_q_pos0, rope_k_pos0):
+      rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm):
     B, H, Sq, D = q.shape
     y = q.new_empty((B, H, Sq, D))
     lse = q.new_empty((B, H, Sq), dtype=torch.float32)
@@ -64,7 +65,8 @@ def _(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scal
 def _bwd_op(dy: Tensor, q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optional[Tensor], v_first: Optional[Tensor],
             vr_coef: Optional[Tensor], gate_logits: Optional[Tensor], y: Tensor, lse: Tensor, kv_ws: Tensor,
             gate_scale: float, eps: float, sm_scale: float, causal: bool, q_start: int,
-            rope_cos: Optional[Tensor], rope_sin: Optional[Tensor], rope_q_pos0: int, rope_k_pos0: int) -> List[Tensor]:
+            rope_cos: Optional[Tensor], rope_sin: Optional[Tensor], rope_q_pos0: int, rope_k_pos0: int,
+            qk_norm: bool) -> List[Tensor]:
     """Returns [dq, dk, dv, dg_q, dg_k, dv_first, dvr_coef, dgate]; absent ones are empty tensors."""
     dev = q.device
     rope = _rope_arg(rope_cos, rope_sin, None if rope_q_pos0 < 0 else rope_q_pos0, rope_k_pos0, q_start, dev, q.shape[-1])
@@ -78,7 +80,8 @@ def _bwd_op(dy: Tensor, q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optio
     dvf = None if v_first is None else torch.empty_like(v_first)
     dgate = None if gate_logits is None else torch.empty_like(gate_logits)
     dg_q, dg_k, dcoef = _backward(q, k, v, gq32, gk32, v_first, c32, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
-                                  y, lse, dy, dq, dk, dv, dvf, dgate, kv_ws, rope)
+                                  y, lse, dy, dq, dk, dv, dvf, dgate, kv_ws, rope,
+                                  0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM)
     none = q.new_empty((0,))
     return [dq, dk, dv, dg_q.reshape(g_q.shape).to(g_q.dtype),
             none if g_k is None else dg_k.reshape(g_k.shape).to(g_k.dtype),
@@ -89,7 +92,7 @@ def _bwd_op(dy: Tensor, q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optio
 
 @_bwd_op.register_fake
 def _(dy, q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, gate_scale, eps, sm_scale, causal, q_start,
-      rope_cos, rope_sin, rope_q_pos0, rope_k_pos0):
+      rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm):
     none = q.new_empty((0,))
     return [torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(g_q),
             none if g_k is None else torch.empty_like(g_k),
@@ -100,22 +103,22 @@ def _(dy, q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, gate_
 
 def _setup_context(ctx, inputs, output):
     (q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
-     rope_cos, rope_sin, rope_q_pos0, rope_k_pos0) = inputs
+     rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm) = inputs
     y, lse, kv_ws = output
     ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, rope_cos, rope_sin)
-    ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start, rope_q_pos0, rope_k_pos0)
+    ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start, rope_q_pos0, rope_k_pos0, qk_norm)
 
 
 def _autograd_backward(ctx, grads):
     dy = grads[0]
     q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, rope_cos, rope_sin = ctx.saved_tensors
-    gate_scale, eps, sm_scale, causal, q_start, rope_q_pos0, rope_k_pos0 = ctx.cfg
+    gate_scale, eps, sm_scale, causal, q_start, rope_q_pos0, rope_k_pos0, qk_norm = ctx.cfg
     dq, dk, dv, dg_q, dg_k, dvf, dcoef, dgate = torch.ops.segpt.qknorm_attention_backward(
         dy, q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, gate_scale, eps, sm_scale, causal, q_start,
-        rope_cos, rope_sin, rope_q_pos0, rope_k_pos0)
+        rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm)
     return (dq, dk, dv, dg_q, None if g_k is None else dg_k, None if v_first is None else dvf,
             None if vr_coef is None else dcoef, None if gate_logits is None else dgate, None, None, None, None, None,
-            None, None, None, None)
+            None, None, None, None, None)
 
 
 _fwd_op.register_autograd(_autograd_backward, setup_context=_setup_context)
@@ -123,12 +126,12 @@ _fwd_op.register_autograd(_autograd_backward, setup_context=_setup_context)
 
 def qknorm_attention_op(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate_logits=None, gate_scale=2.0,
                         eps=1e-6, sm_scale=None, causal=True, q_start=0, return_lse=False,
-                        rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0):
+                        rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0, qk_norm=True):
     """Keyword front end of ``torch.ops.segpt.qknorm_attention`` (same arguments as ``qknorm_attention``)."""
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
     y, lse, _ = torch.ops.segpt.qknorm_attention(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, float(gate_scale),
                                                  float(eps), float(sm_scale), bool(causal), int(q_start),
                                                  rope_cos, rope_sin, -1 if rope_q_pos0 is None else int(rope_q_pos0),
-                                                 int(rope_k_pos0))
+                                                 int(rope_k_pos0), bool(qk_norm))
     return (y, lse) if return_lse else y

@@ -16,8 +16,9 @@ class AttnPlan:
     `backward()` and `backward_stage(i)` then only enqueue kernels on the current stream."""
 
     def __init__(self, x: dict, *, eps=1e-6, sm_scale=None, gate_scale=2.0, causal=True, q_start=0, backward=True,
-                 rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0):
+                 rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0, qk_norm=True):
         self.lib = _lib.load()
+        self.base_flags = 0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM  # part of every call's flags
         q, k, v = x["q"], x["k"], x["v"]
         dev = q.device
         self.x = x
@@ -58,19 +59,19 @@ class AttnPlan:
 
     def forward(self, flags: int = 0):
         """Key/value pre-pass + attention kernel; leaves the normalised keys in the plan's kv workspace."""
-        self.p.flags = flags
+        self.p.flags = flags | self.base_flags
         self._chk(self.lib.segpt_attn_fwd(self.p, self.stream), "segpt_attn_fwd")
 
     def forward_stage(self, stage: int):
-        self.p.flags = 0
+        self.p.flags = self.base_flags
         self._chk(self.lib.segpt_attn_fwd_stage(self.p, stage, self.stream), "segpt_attn_fwd_stage")
 
     def backward(self, kv_prepared: bool = False):
         """`kv_prepared`: forward() ran on this plan since k / v last changed, so the backward reuses its
         normalised keys instead of running the pre-pass again."""
-        self.p.flags = _lib.SEGPT_FLAG_KV_PREPARED if kv_prepared else 0
+        self.p.flags = (_lib.SEGPT_FLAG_KV_PREPARED if kv_prepared else 0) | self.base_flags
         self._chk(self.lib.segpt_attn_bwd(self.p, self.stream), "segpt_attn_bwd")
 
     def backward_stage(self, stage: int, kv_prepared: bool = False):
-        self.p.flags = _lib.SEGPT_FLAG_KV_PREPARED if kv_prepared else 0
+        self.p.flags = (_lib.SEGPT_FLAG_KV_PREPARED if kv_prepared else 0) | self.base_flags
         self._chk(self.lib.segpt_attn_bwd_stage(self.p, stage, self.stream), "segpt_attn_bwd_stage")

@@ -41,7 +41,7 @@ def test_header_constants_match_binding():
     assert int(consts["SEGPT_ABI_VERSION"]) == _lib.SEGPT_ABI_VERSION
     assert int(consts["SEGPT_DTYPE_BF16"]) == _lib.SEGPT_DTYPE_BF16
     assert int(consts["SEGPT_DTYPE_FP32"]) == _lib.SEGPT_DTYPE_FP32
-    for name in ("SEGPT_FLAG_KV_PREPARED", "SEGPT_FLAG_RUNNING_MAX", "SEGPT_FLAG_DECODE", "SEGPT_WS_KV", "SEGPT_WS_BWD"):
+    for name in ("SEGPT_FLAG_KV_PREPARED", "SEGPT_FLAG_RUNNING_MAX", "SEGPT_FLAG_DECODE", "SEGPT_FLAG_NO_NORM", "SEGPT_WS_KV", "SEGPT_WS_BWD"):
         assert int(consts[name]) == getattr(_lib, name), name
     stages = lambda prefix: [k for k, _ in sorted(((k, int(v)) for k, v in consts.items() if k.startswith(prefix)), key=lambda kv: kv[1])]
     assert [s.rsplit("_", 1)[1].lower() for s in stages("SEGPT_FWD_STAGE_")] == list(_lib.FWD_STAGES)
@@ -226,6 +226,6 @@ def test_library_op_is_registered_with_a_shape_only_implementation():
     with FakeTensorMode():  # what torch.compile sees: device tensors without storage
         dev = lambda *s, dt=torch.bfloat16: torch.empty(*s, dtype=dt, device="cuda")
         out = torch.ops.segpt.qknorm_attention(dev(1, 4, 50, 128), dev(1, 2, 70, 128), dev(1, 2, 70, 128), dev(1, dt=torch.float32),
-                                               None, dev(1, 2, 70, 128), dev(2, dt=torch.float32), dev(1, 50, 4), 2.0, 1e-6, 0.1, True, 20, None, None, -1, 0)
+                                               None, dev(1, 2, 70, 128), dev(2, dt=torch.float32), dev(1, 50, 4), 2.0, 1e-6, 0.1, True, 20, None, None, -1, 0, True)
         assert out[0].shape == (1, 4, 50, 128) and out[1].shape == (1, 4, 50)
         assert out[2].numel() == 2 * (2 * 70 * 128 * 2 + 255) // 256 * 256 or out[2].numel() >= 2 * 2 * 70 * 128 * 2

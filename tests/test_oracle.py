@@ -394,3 +394,43 @@ def test_rope_gradients_by_gradcheck():
     cos, sin = orc.rope_tables(8, 10.0, 4)
     fn = lambda q, k, v, gq: orc.attention_forward(q, k, v, gq, None, rope=(cos, sin))[0]
     assert torch.autograd.gradcheck(fn, (q, k, v, gq), eps=1e-6, atol=1e-6)
+
+
+# ------------------------------------------------------------------ attention without QK-norm (plain flash path)
+
+
+def test_plain_variant_is_sdpa_and_the_family_without_normalisers():
+    g = torch.Generator().manual_seed(21)
+    n, S, D = 6, 19, 8
+    Q = 1.7 * torch.randn(n, S, D, generator=g, dtype=F64)  # NOT unit-RMS rows: a stray normaliser would show
+    K = 0.6 * torch.randn(n, S, D, generator=g, dtype=F64)
+    V = torch.randn(n, S, D, generator=g, dtype=F64)
+    out = orc.plain_flash_variant(Q, K, V)
+    assert torch.allclose(out, F.scaled_dot_product_attention(Q, K, V, is_causal=True), atol=1e-12)
+    y = orc.attention_forward(Q[None], K[None], V[None], torch.ones(1, dtype=F64), None, qk_norm=False)[0][0]
+    assert torch.allclose(out, y, atol=1e-12)
+    # with normalisers the result differs (the switch is not a no-op) ...
+    y_n = orc.attention_forward(Q[None], K[None], V[None], torch.ones(1, dtype=F64), None)[0][0]
+    assert (y_n - out).abs().max() > 1e-2
+    # ... and scaling a query row now changes the logits (no scale invariance left)
+    Q2 = Q.clone()
+    Q2[:, 5] *= 3.0
+    assert (orc.plain_flash_variant(Q2, K, V)[:, 5] - out[:, 5]).abs().max() > 1e-3
+    # q_start / non-causal arguments (note the order: q_start, is_causal -- triton_flash_attn.py:215-216)
+    full = orc.plain_flash_variant(Q, K, V, 0, True)
+    tail = orc.plain_flash_variant(Q[:, 12:], K, V, 12, True)
+    assert torch.allclose(tail, full[:, 12:], atol=1e-12)
+    assert torch.allclose(orc.plain_flash_variant(Q, K, V, 0, False), F.scaled_dot_product_attention(Q, K, V), atol=1e-12)
+
+
+@pytest.mark.parametrize("extras", [False, True])
+def test_plain_explicit_backward_matches_autograd(extras):
+    q, k, v, gq, gk, dy, kw = _bwd_case(extras)
+    q = 1.5 * q
+    ex = orc.attention_backward_explicit(q, k, v, gq, gk, dy, qk_norm=False, **kw)
+    ag = orc.attention_backward_autograd(q, k, v, gq, gk, dy, qk_norm=False, **kw)
+    for name in ag:
+        assert torch.allclose(ex[name], ag[name], atol=1e-10), name
+    # against the normalised family the gradients differ
+    ex_n = orc.attention_backward_explicit(q, k, v, gq, gk, dy, **kw)
+    assert (ex_n["dq"] - ex["dq"]).abs().max() > 1e-3

@@ -9,7 +9,8 @@ import pytest
 import torch
 
 from oracle import qknorm_attn_oracle as orc
-from sample_efficient_gpt_amd import CONFIGS, QKNormFlashAttnFunc, SelfDotProductAttnQKNorm, make_inputs, qknorm_attention
+from sample_efficient_gpt_amd import (CONFIGS, FlashAttnFunc, QKNormFlashAttnFunc, SelfDotProductAttnQKNorm, make_inputs,
+                                      qknorm_attention, qknorm_attention_op)
 from tests.parity_util import compare, gen, run_gpu, run_oracle, scalar_gain_scale
 
 pytestmark = pytest.mark.gpu
@@ -244,7 +245,7 @@ def test_library_op_compiled_and_checkpointed_matches_eager(gpu_device):
         for a, b in zip(ref, other):
             assert torch.equal(a, b)
     torch.library.opcheck(torch.ops.segpt.qknorm_attention,
-                          tuple(x[n].to(gpu_device) for n in names) + (2.0, 1e-6, 0.125, True, 0, None, None, -1, 0),
+                          tuple(x[n].to(gpu_device) for n in names) + (2.0, 1e-6, 0.125, True, 0, None, None, -1, 0, True),
                           test_utils=("test_schema", "test_faketensor"))
 
 
@@ -325,6 +326,66 @@ def test_decode_path_matches_oracle_and_training_kernel(gpu_device, B, H, Hkv, S
     compare({n: trn[n] for n in ("y", "lse")}, ref, BF16)
     assert torch.allclose(dec["y"].float(), trn["y"].float(), atol=2e-2, rtol=1e-2)
     assert torch.allclose(dec["lse"], trn["lse"], atol=2e-2, rtol=1e-2)
+
+
+# ------------------------------------------------------------------ attention without QK-norm (SEGPT_FLAG_NO_NORM)
+
+
+@pytest.mark.parametrize(
+    "dtype,B,H,Hkv,Sq,Sk,D,kw,gen_kw",
+    [
+        (F32, 2, 4, 2, 130, 130, 64, {}, {"scalar_gain": True, "no_gk": True}),
+        (F32, 1, 3, 3, 40, 104, 128, {"q_start": 64}, {"extras": True}),
+        (BF16, 2, 6, 2, 384, 384, 64, {}, {"scalar_gain": True, "no_gk": True}),
+        (BF16, 1, 3, 1, 300, 300, 64, {}, {}),                           # the scale vectors still apply
+        (BF16, 1, 4, 2, 200, 200, 64, {"gate_scale": 2.0}, {"extras": True}),
+        (BF16, 1, 2, 1, 256, 256, 128, {}, {"head_scales": True}),       # rows of different norms: logits up to +-20
+        (BF16, 1, 2, 2, 96, 200, 64, {"causal": False}, {}),
+        (BF16, 1, 3, 3, 72, 200, 64, {"q_start": 128}, {}),
+    ],
+)
+def test_plain_attention_fwd_bwd(gpu_device, dtype, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
+    """qk_norm=False: normalisers fixed at 1, against the oracle's family with the same switch (itself pinned
+    against SDPA).  head_scales makes the row norms differ, so a normaliser left in by mistake would show."""
+    _case(gpu_device, dtype, B, H, Hkv, Sq, Sk, D, gen_kw=gen_kw, qk_norm=False, **kw)
+
+
+def test_plain_dropin_matches_sdpa_restatement(gpu_device):
+    """FlashAttnFunc.apply(Q, K, V, q_start, is_causal) -- the reference's TritonFlashAttnFunc call shape
+    (attention.py:240) -- against the brute-force softmax restatement and its autograd gradients; GQA-native
+    K/V equal the expanded call; the library op reaches the same kernels."""
+    B, H, Hkv, S, D = 2, 6, 2, 320, 64
+    x = gen(B, H, Hkv, S, S, D, BF16, seed=17, head_scales=True)
+    x["q"] = (x["q"].float() * 0.7).to(BF16)
+    Q, K, V, dO = _flat(x["q"], H), _flat(x["k"], Hkv), _flat(x["v"], Hkv), _flat(x["d_o"], H)
+    Kx, Vx = (orc.expand_kv_flat(t, Hkv, H).contiguous() for t in (K, V))
+    Qr, Kr, Vr = (t.detach().clone().double().requires_grad_(True) for t in (Q, Kx, Vx))
+    ref_out = orc.plain_flash_variant(Qr, Kr, Vr, 0, True)
+    ref_out.backward(dO.double())
+    d = gpu_device
+    Qd, Kd, Vd = (t.detach().clone().to(d).requires_grad_(True) for t in (Q, Kx, Vx))
+    out = FlashAttnFunc.apply(Qd, Kd, Vd, 0, True)
+    assert out.shape == Q.shape and out.dtype == Q.dtype
+    out.backward(dO.to(d))
+    got = {"y": out.detach().cpu(), "dq": Qd.grad.cpu(), "dk": Kd.grad.cpu(), "dv": Vd.grad.cpu()}
+    ref = {"y": ref_out.detach(), "dq": Qr.grad, "dk": Kr.grad, "dv": Vr.grad}
+    print("plain drop-in max abs err", compare(got, ref, BF16), flush=True)
+    # un-expanded GQA tensors: same output bits, dK/dV are the group sums
+    Qn, Kn, Vn = (t.detach().clone().to(d).requires_grad_(True) for t in (Q, K, V))
+    o_nat = FlashAttnFunc.apply(Qn, Kn, Vn, 0, True, Hkv)
+    assert torch.equal(o_nat, out)
+    o_nat.backward(dO.to(d))
+    rep = H // Hkv
+    dk_sum = ref["dk"].reshape(Hkv, rep, B, S, D).sum(1).reshape(Hkv * B, S, D)
+    compare({"dk": Kn.grad.cpu()}, {"dk": dk_sum}, BF16)
+    # decode-time call shape: q_start = past length, forward only (split-key kernels)
+    with torch.no_grad():
+        tail = FlashAttnFunc.apply(Q[:, 317:].contiguous().to(d), K.to(d), V.to(d), 317, True, Hkv)
+    compare({"y": tail.cpu()}, {"y": ref_out.detach()[:, 317:]}, BF16)
+    # the registered op with qk_norm=False
+    q4 = x["q"].to(d)
+    y_op = qknorm_attention_op(q4, x["k"].to(d), x["v"].to(d), torch.ones(1, device=d), None, qk_norm=False)
+    assert torch.equal(orc.flatten_heads(y_op.cpu()), out.detach().cpu())
 
 
 def test_backward_is_deterministic(gpu_device):
