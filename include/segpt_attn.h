@@ -56,7 +56,7 @@ extern "C" {
 #define SEGPT_E_EXTRAS -8      /* v_first without vr_coef or the reverse; missing grad slot */
 #define SEGPT_E_QSTART -9      /* q_start < 0                                               */
 #define SEGPT_E_ALIGN -10      /* a base pointer is not 16-byte aligned                     */
-#define SEGPT_E_ROPE -12       /* rope tables: one NULL, misaligned, too short for the positions, or fp32 dtype */
+#define SEGPT_E_ROPE -12       /* rope tables: one NULL, misaligned, or too short for the positions */
 #define SEGPT_E_STAGE -11      /* unknown stage passed to segpt_attn_bwd_stage              */
 
 /* segpt_attn_params.flags */
@@ -156,7 +156,7 @@ typedef struct segpt_attn_params {
 
   /* optional rotary embedding of q and k, fused into the loads (the step before the op in the reference:
    * rope.py:36-56 applied at attention.py:202-204).  Split-half pairs (j, j + D/2); query row i uses table row
-   * rope_q_pos0 + i, key row j uses rope_k_pos0 + j.  Both tables or neither; bf16 only.  dq / dk are
+   * rope_q_pos0 + i, key row j uses rope_k_pos0 + j.  Both tables or neither.  dq / dk are
    * gradients with respect to the UNROTATED inputs. */
   const float* rope_cos; /* [rope_len, D/2] fp32 device, 16 B aligned, or NULL */
   const float* rope_sin; /* [rope_len, D/2] fp32 device, 16 B aligned, or NULL */

@@ -98,7 +98,7 @@ int check_common(const segpt_attn_params* p) {
   if (p->v_first.ptr && (rc = check_t4(p->v_first, *p))) return rc;
   if (p->gate.ptr && (p->gate.stride_b < 0 || p->gate.stride_s < 0 || p->gate.stride_h < 0)) return SEGPT_E_STRIDE;
   if (p->rope_cos || p->rope_sin) {
-    if (!p->rope_cos || !p->rope_sin || p->dtype != SEGPT_DTYPE_BF16) return SEGPT_E_ROPE;
+    if (!p->rope_cos || !p->rope_sin) return SEGPT_E_ROPE;
     if (!aligned16(p->rope_cos) || !aligned16(p->rope_sin)) return SEGPT_E_ROPE;
     if (p->rope_q_pos0 < 0 || p->rope_k_pos0 < 0) return SEGPT_E_ROPE;
     if ((int64_t)p->rope_q_pos0 + p->Sq > p->rope_len || (int64_t)p->rope_k_pos0 + p->Sk > p->rope_len) return SEGPT_E_ROPE;
@@ -164,7 +164,7 @@ const char* segpt_strerror(int code) {
     case SEGPT_E_EXTRAS: return "inconsistent optional operands (v_first/vr_coef/gate and their gradient slots)";
     case SEGPT_E_QSTART: return "q_start must be >= 0";
     case SEGPT_E_ALIGN: return "a base pointer is not 16-byte aligned (workspace: 256-byte)";
-    case SEGPT_E_ROPE: return "rope tables: both or neither, 16-byte aligned, rope_len >= position + rows, bf16 only";
+    case SEGPT_E_ROPE: return "rope tables: both or neither, 16-byte aligned, rope_len >= position + rows";
     case SEGPT_E_STAGE: return "unknown stage (expected SEGPT_FWD_STAGE_* / SEGPT_BWD_STAGE_*)";
     default: return code > 0 ? "HIP runtime error raised by a kernel launch" : "unknown segpt error code";
   }

@@ -26,6 +26,25 @@ __device__ __forceinline__ float oct_sum(float x) {
   return x;
 }
 
+// Split-half rotary embedding (rope.py:50-55) of a row spread over TPR consecutive lanes, N = D/TPR contiguous
+// elements per lane starting at d0 = (lane % TPR) * N: the partner element d +- D/2 sits TPR/2 lanes away at
+// the same index.  `pos` is the row's table row.  Every lane of the wave must get here (the lanes shuffle).
+// INVERSE applies the transpose, i.e. takes a gradient in the rotated frame back to the unrotated row.
+template <int D, int N, int TPR, bool INVERSE>
+__device__ __forceinline__ void rope_lanes(const segpt_attn_params& p, float (&x)[N], int pos, int d0) {
+  static_assert(N * TPR == D, "row split");
+  const bool hi = d0 >= D / 2;
+  const float* cosr = p.rope_cos + (int64_t)pos * (D / 2) + (hi ? d0 - D / 2 : d0);
+  const float* sinr = p.rope_sin + (int64_t)pos * (D / 2) + (hi ? d0 - D / 2 : d0);
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    const float o = __shfl_xor(x[e], TPR / 2, 64);
+    const float c = cosr[e];
+    const float sn = INVERSE ? -sinr[e] : sinr[e];
+    x[e] = hi ? o * sn + x[e] * c : x[e] * c - o * sn;
+  }
+}
+
 template <int D>
 __device__ __forceinline__ float gprod(const segpt_attn_params& p, int d) {
   float gq = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
@@ -68,6 +87,7 @@ __device__ __forceinline__ void stage_kv(const segpt_attn_params& p, int b, int 
 #pragma unroll
     for (int e = 0; e < PT; ++e) { kreg[e] = 0.f; vreg[e] = 0.f; }
   }
+  if (p.rope_cos) rope_lanes<D, PT, 8, false>(p, kreg, p.rope_k_pos0 + min(j, p.Sk - 1), part * PT);
   float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < PT; ++e) ss += kreg[e] * kreg[e];
@@ -98,14 +118,17 @@ __global__ __launch_bounds__(kThreads) void fwd_f32_kernel(KArgs a) {
   float qh[DP], acc[DP];
   {
     const float* qp = row_ptr<float>(p.q, b, h, rowc) + sub * DP;
-    float ss = 0.f;
 #pragma unroll
     for (int e = 0; e < DP; e += 4) {
       float t[4];
       Elem<float>::load(qp + e, t);
 #pragma unroll
-      for (int x = 0; x < 4; ++x) { qh[e + x] = t[x]; ss += t[x] * t[x]; }
+      for (int x = 0; x < 4; ++x) qh[e + x] = t[x];
     }
+    if (p.rope_cos) rope_lanes<D, DP, 4, false>(p, qh, p.rope_q_pos0 + rowc, sub * DP);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < DP; ++e) ss += qh[e] * qh[e];
     ss = quad_sum(ss);
     const float alpha = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
@@ -194,17 +217,21 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_f32_kernel(KArgs a) {
     const float* qp = row_ptr<float>(p.q, b, h, rowc) + sub * DP;
     const float* dp = a.do_eff ? reinterpret_cast<const float*>(a.do_eff) + (((int64_t)b * p.H + h) * p.Sq + rowc) * D + sub * DP
                                : row_ptr<float>(p.d_o, b, h, rowc) + sub * DP;
-    float ss = 0.f;
 #pragma unroll
     for (int e = 0; e < DP; e += 4) {
       float t[4];
       Elem<float>::load(qp + e, t);
 #pragma unroll
-      for (int x = 0; x < 4; ++x) { qraw[e + x] = t[x]; ss += t[x] * t[x]; }
+      for (int x = 0; x < 4; ++x) qraw[e + x] = t[x];
       Elem<float>::load(dp + e, t);
 #pragma unroll
       for (int x = 0; x < 4; ++x) dout[e + x] = t[x];
     }
+    // with a rotary embedding qraw is the ROTATED row from here on: the normaliser and the scale act on it
+    if (p.rope_cos) rope_lanes<D, DP, 4, false>(p, qraw, p.rope_q_pos0 + rowc, sub * DP);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < DP; ++e) ss += qraw[e] * qraw[e];
     ss = quad_sum(ss);
     alpha = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
@@ -249,15 +276,18 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_f32_kernel(KArgs a) {
     dgl[e] = live ? p.sm_scale * alpha * qraw[e] * T[e] : 0.f;
   }
   dot = quad_sum(dot);
-  if (live) {
+  {
     const float a3 = norm_grad_coef(p, alpha, 1.0f / D) * dot;
-    float* op = row_ptr_mut<float>(p.dq, b, h, row) + sub * DP;
 #pragma unroll
-    for (int e = 0; e < DP; e += 4) {
-      float t[4];
+    for (int e = 0; e < DP; ++e) u[e] = alpha * u[e] - a3 * qraw[e];  // gradient of the (rotated) row
+    if (p.rope_cos) rope_lanes<D, DP, 4, true>(p, u, p.rope_q_pos0 + rowc, sub * DP);
+    if (live) {
+      float* op = row_ptr_mut<float>(p.dq, b, h, row) + sub * DP;
 #pragma unroll
-      for (int x = 0; x < 4; ++x) t[x] = alpha * u[e + x] - a3 * qraw[e + x];
-      Elem<float>::store(op + e, t);
+      for (int e = 0; e < DP; e += 4) {
+        float t[4] = {u[e], u[e + 1], u[e + 2], u[e + 3]};
+        Elem<float>::store(op + e, t);
+      }
     }
   }
   // block partial of dg: sum over the 16 rows of a wave (lanes with equal sub), then over 4 waves
@@ -311,7 +341,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkdv_f32_kernel(KArgs a) {
       float t[4];
       Elem<float>::load(kp + e, t);
 #pragma unroll
-      for (int x = 0; x < 4; ++x) { kh[e + x] = t[x]; ss += t[x] * t[x]; }
+      for (int x = 0; x < 4; ++x) kh[e + x] = t[x];
       Elem<float>::load(vp + e, t);
 #pragma unroll
       for (int x = 0; x < 4; ++x) vmix[e + x] = t[x];
@@ -326,6 +356,9 @@ __global__ __launch_bounds__(kThreads) void bwd_dkdv_f32_kernel(KArgs a) {
         for (int x = 0; x < 4; ++x) vmix[e + x] = c1 * vmix[e + x] + c2 * t[x];
       }
     }
+    if (p.rope_cos) rope_lanes<D, DP, 4, false>(p, kh, p.rope_k_pos0 + jc, sub * DP);
+#pragma unroll
+    for (int e = 0; e < DP; ++e) ss += kh[e] * kh[e];
     ss = quad_sum(ss);
     beta = row_normaliser(p, ss, 1.0f / D);
 #pragma unroll
@@ -361,6 +394,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkdv_f32_kernel(KArgs a) {
 #pragma unroll
           for (int e = 0; e < PT; ++e) { qreg[e] = 0.f; dreg[e] = 0.f; }
         }
+        if (p.rope_cos) rope_lanes<D, PT, 8, false>(p, qreg, p.rope_q_pos0 + min(i, p.Sq - 1), part * PT);
         float ss = 0.f;
 #pragma unroll
         for (int e = 0; e < PT; ++e) ss += qreg[e] * qreg[e];
@@ -406,19 +440,27 @@ __global__ __launch_bounds__(kThreads) void bwd_dkdv_f32_kernel(KArgs a) {
       float t[4];
       Elem<float>::load(kp + e, t);
 #pragma unroll
-      for (int x = 0; x < 4; ++x) { kraw[e + x] = t[x]; dot += W[e + x] * t[x]; }
+      for (int x = 0; x < 4; ++x) kraw[e + x] = t[x];
     }
   }
+  if (p.rope_cos) rope_lanes<D, DP, 4, false>(p, kraw, p.rope_k_pos0 + jc, sub * DP);  // the normaliser saw the rotated row
+#pragma unroll
+  for (int e = 0; e < DP; ++e) dot += W[e] * kraw[e];
   dot = quad_sum(dot);
-  if (live) {
+  {
     const float b3 = norm_grad_coef(p, beta, 1.0f / D) * dot;
+#pragma unroll
+    for (int e = 0; e < DP; ++e) W[e] = beta * W[e] - b3 * kraw[e];
+    if (p.rope_cos) rope_lanes<D, DP, 4, true>(p, W, p.rope_k_pos0 + jc, sub * DP);
+  }
+  if (live) {
     float* okp = row_ptr_mut<float>(p.dk, b, g, j) + sub * DP;
     float* ovp = row_ptr_mut<float>(p.dv, b, g, j) + sub * DP;
 #pragma unroll
     for (int e = 0; e < DP; e += 4) {
       float t[4];
 #pragma unroll
-      for (int x = 0; x < 4; ++x) t[x] = beta * W[e + x] - b3 * kraw[e + x];
+      for (int x = 0; x < 4; ++x) t[x] = W[e + x];
       Elem<float>::store(okp + e, t);
 #pragma unroll
       for (int x = 0; x < 4; ++x) t[x] = c1 * dV[e + x];

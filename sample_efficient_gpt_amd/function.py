@@ -196,7 +196,7 @@ def qknorm_attention(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate
     aligned); g_q, g_k scale parameters of 1 or D elements; vr_coef device tensor ``[2]`` = (c1, c2)
     with ``v' = c1 v + c2 v_first``; gate_logits ``[B,Sq,H]`` with ``y = gate_scale*sigmoid(z)*o``.
     rope_cos / rope_sin ``[len, D/2]``: q and k are the UNROTATED projections and the split-half rotary
-    embedding (rope.py:36-56) is applied inside the kernels' loads (bf16 only); query row i sits at position
+    embedding (rope.py:36-56) is applied inside the kernels' loads; query row i sits at position
     ``rope_q_pos0 + i`` (default ``q_start``), key row j at ``rope_k_pos0 + j``.
     ``qk_norm=False``: no RMS normalisation of q and k (eps unused) -- the reference's attention without QK-norm
     (attention.py:233-240); the scale vectors still apply, pass ``g_q = ones(1)`` for the plain op.

@@ -116,8 +116,8 @@ def test_argument_errors_are_reported_before_any_launch(lib):
     assert lib.segpt_attn_fwd(p, None) == -12
     p.rope_q_pos0, p.rope_sin = 0, 0x60004
     assert lib.segpt_attn_fwd(p, None) == -12
-    p = _valid_params(dtype=_lib.SEGPT_DTYPE_FP32); p.rope_cos, p.rope_sin, p.rope_len = 0x50000, 0x60000, 4096
-    assert lib.segpt_attn_fwd(p, None) == -12
+    p = _valid_params(dtype=_lib.SEGPT_DTYPE_FP32); p.rope_cos, p.rope_sin, p.rope_len = 0x50000, 0x60000, p.Sk - 1
+    assert lib.segpt_attn_fwd(p, None) == -12  # the fp32 path takes the tables too, under the same checks
     # backward-only checks
     p = _valid_params()
     assert lib.segpt_attn_bwd(p, None) == -7  # no workspace

@@ -285,9 +285,24 @@ def test_fused_rope_equals_rotating_first_and_rejects_bad_tables(gpu_device):
     short = orc.rope_tables(100, 10000.0, 64)
     with pytest.raises(_lib.SegptError):  # table shorter than the positions it must serve
         run_gpu(x, gpu_device, backward=False, rope=short)
-    xf = gen(1, 2, 2, 64, 64, 64, F32, seed=1)
-    with pytest.raises(_lib.SegptError):  # the fp32 path has no fused rotary embedding
-        run_gpu(xf, gpu_device, backward=False, rope=(cos, sin))
+
+
+@pytest.mark.parametrize(
+    "B,H,Hkv,Sq,Sk,D,kw,gen_kw",
+    [
+        (2, 4, 2, 130, 130, 64, {}, {}),
+        (1, 6, 2, 100, 100, 64, {}, {"extras": True}),
+        (1, 2, 1, 77, 77, 32, {}, {"scalar_gain": True, "no_gk": True}),
+        (1, 4, 1, 70, 70, 128, {}, {}),
+        (1, 3, 3, 40, 104, 64, {"q_start": 64}, {}),                      # query positions start at q_start
+        (1, 2, 2, 48, 80, 64, {"causal": False, "rope_q_pos0": 11, "rope_k_pos0": 3}, {}),
+        (1, 2, 1, 64, 64, 64, {"qk_norm": False}, {"scalar_gain": True, "no_gk": True}),
+    ],
+)
+def test_fp32_fused_rope(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
+    """The rotary embedding on the fp32 parity path: forward, dq and dk (gradients with respect to the UNROTATED
+    rows) against the oracle at 1e-5 -- pins the pair indexing and the table rows far tighter than bf16 can."""
+    _case(gpu_device, F32, B, H, Hkv, Sq, Sk, D, gen_kw=gen_kw, rope=orc.rope_tables(160, 10000.0, D), **kw)
 
 
 # ------------------------------------------------------------------ decode-shaped calls (split-key kernels)
