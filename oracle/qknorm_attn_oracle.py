@@ -15,6 +15,8 @@ reference computes on its attention path:
 * the attention without QK-norm, `attention.py:233-240` (SDPA) and `TritonFlashAttnFunc`,
   `sample_efficient_gpt/transformer/ops/triton_flash_attn.py:208-297`   -> ``plain_flash_variant``
   (the family with ``qk_norm=False``)
+* the whole module `MultiHeadSelfAttention.forward`, `attention.py:175-267` (projection, RoPE, GQA
+  expansion, KV cache, value residual, attention, gate, output projection)   -> ``mhsa_forward``
 * the caller glue of `attention.py:199-255`: `(h b)` head-major flatten, GQA
   `repeat_interleave`, value-residual mix, per-head `2*sigmoid` gate
                                                           -> ``flatten_heads`` ... ``caller_glue``
@@ -37,6 +39,9 @@ this path, so every pin is mathematical -- see tests/test_oracle.py):
 * ``plain_flash_variant``   pinned against ``F.scaled_dot_product_attention`` and the family with
   ``qk_norm=False``; the ``qk_norm=False`` explicit backward against autograd in fp64.
 * layout helpers           pinned by brute-force python indexing on tiny tensors.
+* ``mhsa_forward``          the whole module forward (attention.py:175-267) in the reference's flattened
+  layouts; pinned against the separately written ``caller_glue`` + ``apply_rope`` composition, a per-(batch,
+  head) python loop over plain softmax attention, and prefill + cached single-token steps == one full pass.
 
 The exact bf16 rounding order of variant A (normalise -> round -> times
 bf16(gain) -> round, attention.py:59-62) is restated in ``live_module_variant_a``
@@ -337,15 +342,16 @@ def live_module_variant_a(Q, K, V, gain, is_causal: bool = True, q_start: int = 
     fp32 so that it also runs for bf16 inputs on CPU without a fused backend.
     """
     eps = 1e-6
-    qf, kf = Q.float(), K.float()
+    ct = torch.float64 if Q.dtype == torch.float64 else torch.float32  # fp64 callers keep their precision
+    qf, kf = Q.to(ct), K.to(ct)
     qn = (qf * rms_inv(qf, eps)).to(Q.dtype)
     kn = (kf * rms_inv(kf, eps)).to(K.dtype)
     qn = qn * gain.to(qn.dtype)
     d = Q.shape[-1]
-    s = torch.einsum("nid,njd->nij", qn.float(), kn.float()) / math.sqrt(d)
+    s = torch.einsum("nid,njd->nij", qn.to(ct), kn.to(ct)) / math.sqrt(d)
     vis = visibility_mask(Q.shape[-2], K.shape[-2], is_causal, q_start)
     s = s.masked_fill(~vis, float("-inf"))
-    return (torch.softmax(s, dim=-1) @ V.float()).to(Q.dtype)
+    return (torch.softmax(s, dim=-1) @ V.to(ct)).to(Q.dtype)
 
 
 def fused_kernel_variant_b(Q, K, V, gain, is_causal: bool = True, q_start: int = 0):
@@ -446,3 +452,71 @@ def caller_glue(q, k, v, gain, *, v1=None, alpha1=None, alpha2=None, scale=None,
     if gate_logits is not None:
         attn = (2.0 * torch.sigmoid(gate_logits)).unsqueeze(-1) * attn
     return attn.reshape(B, S, H * D), V
+
+
+# --------------------------------------------------------------------------- the whole attention module
+
+
+def mhsa_forward(x, w, *, n_heads, n_kv_heads=None, theta=10000.0, max_seq_len=4096, qknorm=True, gating=False,
+                 v1=None, cache=None, rope=None):
+    """`MultiHeadSelfAttention.forward`, attention.py:175-267, step by step in the reference's own layouts.
+
+    x [b, S, d_model]; `w` holds the weights under the reference's state-dict names: ``qkv.linear.weight``
+    [(H+2Hkv)d, d_model], ``out.linear.weight`` [d_model, d_model] (bias-free Linear, core.py:18),
+    ``sdpa_qknorm.gain`` [1] when qknorm, ``alpha1`` / ``alpha2`` / ``scale`` [1] (absent: the buffers 1, 0, 1 of
+    attention.py:154-159), ``attn_gate.linear.weight`` when gating ("elementwise" / "per-head" / "per-head-hd",
+    attention.py:162-171).  `cache`: None or a dict with "keys" / "values" (None or the flattened, head-expanded,
+    ROTATED keys and raw values KVCache holds, attention.py:15-27); it is updated like `KVCache.append`.
+    `rope`: (cos, sin) tables to use instead of building them from theta (e.g. the fp32 tables of the module under
+    test, rope.py:12-24 computes them in fp32).
+    Returns (attn_out [b, S, d_model], V [(h b), Sk, d]) -- V is the mixed, expanded value tensor the
+    reference hands to later layers (attention.py:267).
+    """
+    b, S, d_model = x.shape
+    H = n_heads
+    Hkv = H if n_kv_heads is None else n_kv_heads
+    d = d_model // H
+    q_out, kv_out = H * d, Hkv * d
+    proj = x @ w["qkv.linear.weight"].T                                           # :180
+    Q, K, V = proj[..., :q_out], proj[..., q_out:q_out + kv_out], proj[..., q_out + kv_out:]
+    past = 0
+    if cache is not None and cache.get("keys") is not None:
+        past = cache["keys"].shape[1]                                             # :186
+    q_start = past if cache is not None else 0
+    Q = flatten_heads(Q.reshape(b, S, H, d).permute(0, 2, 1, 3))                  # :199 "b seq (h head_d) -> (h b) seq head_d"
+    K = flatten_heads(K.reshape(b, S, Hkv, d).permute(0, 2, 1, 3))
+    cos, sin = rope if rope is not None else rope_tables(
+        max_seq_len, theta, d, dtype=torch.float64 if x.dtype == torch.float64 else torch.float32)
+    Q = apply_rope(Q, cos, sin, q_start)                                          # :202-204, positions past .. past+S-1
+    K = apply_rope(K, cos, sin, q_start)
+    if Hkv != H:
+        K = expand_kv_flat(K, Hkv, H)                                             # :207-211
+    V = flatten_heads(V.reshape(b, S, Hkv, d).permute(0, 2, 1, 3))                # :213
+    if Hkv != H:
+        V = expand_kv_flat(V, Hkv, H)
+    if cache is not None:                                                         # :220-221 / KVCache.append
+        if cache.get("keys") is not None:
+            K, V = torch.cat((cache["keys"], K), dim=1), torch.cat((cache["values"], V), dim=1)
+        cache["keys"], cache["values"] = K, V
+    V1 = V if v1 is None else v1.reshape(V.shape)                                 # :222-225
+    one, zero = torch.ones(1, dtype=x.dtype), torch.zeros(1, dtype=x.dtype)
+    a1, a2, sc = w.get("alpha1", one), w.get("alpha2", zero), w.get("scale", one)
+    V = sc * (a1 * V + a2 * V1) * torch.rsqrt(a1**2 + a2**2 + 1e-8)               # :228
+    if qknorm:
+        attn = live_module_variant_a(Q, K, V, w["sdpa_qknorm.gain"], True, q_start)   # :232
+    else:
+        attn = plain_flash_variant(Q, K, V, q_start, True)                        # :236 / :240
+    attn = attn.reshape(H, b, S, d).permute(1, 2, 0, 3)                           # b seq h head_d
+    if not gating:
+        attn_cat = attn.reshape(b, S, H * d)                                      # :243
+    elif gating == "elementwise":
+        attn_cat = (2.0 * torch.sigmoid(x @ w["attn_gate.linear.weight"].T)) * attn.reshape(b, S, H * d)   # :246-248
+    elif gating == "per-head":
+        gate = (2.0 * torch.sigmoid(x @ w["attn_gate.linear.weight"].T)).unsqueeze(-1)                   # :251
+        attn_cat = (gate * attn).reshape(b, S, H * d)
+    elif gating == "per-head-hd":
+        gate = (2.0 * torch.sigmoid(x[..., :d] @ w["attn_gate.linear.weight"].T)).unsqueeze(-1)          # :259
+        attn_cat = (gate * attn).reshape(b, S, H * d)
+    else:
+        raise ValueError(f"gating={gating!r} is undefined")
+    return attn_cat @ w["out.linear.weight"].T, V                                 # :265-267

@@ -8,7 +8,7 @@ through the C ABI of ``libsegpt_attn.so``; there is no fallback path.
 """
 
 from .function import FlashAttnFunc, QKNormFlashAttnFunc, qknorm_attention  # noqa: F401
-from .module import SelfDotProductAttnQKNorm  # noqa: F401
+from .module import KVCache, MultiHeadSelfAttention, SelfDotProductAttnQKNorm  # noqa: F401
 from .library_op import qknorm_attention_op  # noqa: F401  (registers torch.ops.segpt.qknorm_attention)
 from .inputs import CONFIGS, AttnConfig, make_inputs  # noqa: F401
 

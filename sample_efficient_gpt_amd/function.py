@@ -146,7 +146,7 @@ class _CoreFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope=None,
-                flags=0):
+                flags=0, out_bshd=False):
         gq32, gk32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device)
         coef32 = None if vr_coef is None else vr_coef.detach().to(device=q.device, dtype=torch.float32).reshape(-1).contiguous()
         _check_inputs(q, k, v, gq32, gk32, v_first, coef32, gate)
@@ -154,9 +154,13 @@ class _CoreFunc(torch.autograd.Function):
         v_first = None if v_first is None else _lastdim_contig(v_first)
         if sm_scale is None:
             sm_scale = 1.0 / math.sqrt(q.shape[-1])
-        y = torch.empty_like(q)
-        if y.stride(-1) != 1:
-            y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        if out_bshd:  # [B,H,Sq,D] view of a [B,Sq,H,D] buffer: the layout the output projection consumes
+            B, H, Sq, D = q.shape
+            y = torch.empty((B, Sq, H, D), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
+        else:
+            y = torch.empty_like(q)
+            if y.stride(-1) != 1:
+                y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope,
                               inference=not any(ctx.needs_input_grad), flags=flags)
         # the normalised keys (bf16 path) are kept for the backward: 1/rep of q's size
@@ -184,12 +188,12 @@ class _CoreFunc(torch.autograd.Function):
             dg_k = dg_k.reshape(g_k.shape).to(g_k.dtype)
         if vr_coef is not None:
             dcoef = dcoef.reshape(vr_coef.shape).to(vr_coef.dtype)
-        return dq, dk, dv, dg_q, dg_k, dv_first, dcoef, dgate, None, None, None, None, None, None, None
+        return dq, dk, dv, dg_q, dg_k, dv_first, dcoef, dgate, None, None, None, None, None, None, None, None
 
 
 def qknorm_attention(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate_logits=None, gate_scale=2.0,
                      eps=1e-6, sm_scale=None, causal=True, q_start=0, return_lse=False,
-                     rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0, qk_norm=True):
+                     rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0, qk_norm=True, out_bshd=False):
     """Fused QK-norm attention on canonical views.
 
     q ``[B,H,Sq,D]``; k, v, v_first ``[B,Hkv,Sk,D]`` (any strides, last dim contiguous, rows 16 B
@@ -200,10 +204,12 @@ def qknorm_attention(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate
     ``rope_q_pos0 + i`` (default ``q_start``), key row j at ``rope_k_pos0 + j``.
     ``qk_norm=False``: no RMS normalisation of q and k (eps unused) -- the reference's attention without QK-norm
     (attention.py:233-240); the scale vectors still apply, pass ``g_q = ones(1)`` for the plain op.
+    ``out_bshd=True``: the returned ``[B,H,Sq,D]`` tensor is a view of a ``[B,Sq,H,D]`` buffer, so that
+    ``y.permute(0, 2, 1, 3).reshape(B, Sq, H*D)`` is the ``b seq (h head_d)`` tensor of attention.py:243 without a copy.
     """
     rope = _rope_arg(rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, q_start, q.device, q.shape[-1])
     y, lse = _CoreFunc.apply(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
-                             rope, 0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM)
+                             rope, 0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM, out_bshd)
     return (y, lse) if return_lse else y
 
 

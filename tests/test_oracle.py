@@ -434,3 +434,96 @@ def test_plain_explicit_backward_matches_autograd(extras):
     # against the normalised family the gradients differ
     ex_n = orc.attention_backward_explicit(q, k, v, gq, gk, dy, **kw)
     assert (ex_n["dq"] - ex["dq"]).abs().max() > 1e-3
+
+
+# ------------------------------------------------------------------ the whole module (attention.py:175-267)
+
+
+def _mhsa_weights(d_model, H, Hkv, gating, value_residual, qknorm, seed=5):
+    g = torch.Generator().manual_seed(seed)
+    d = d_model // H
+    r = lambda *s: torch.randn(*s, generator=g, dtype=F64)
+    w = {"qkv.linear.weight": r((H + 2 * Hkv) * d, d_model) / math.sqrt(d_model), "out.linear.weight": r(d_model, d_model) / math.sqrt(d_model)}
+    if qknorm:
+        w["sdpa_qknorm.gain"] = torch.tensor([1.3], dtype=F64)
+    if value_residual:
+        w.update(alpha1=torch.tensor([0.8], dtype=F64), alpha2=torch.tensor([0.5], dtype=F64), scale=torch.tensor([1.1], dtype=F64))
+    if gating:
+        shape = {"elementwise": (d_model, d_model), "per-head": (H, d_model), "per-head-hd": (H, d)}[gating]
+        w["attn_gate.linear.weight"] = r(*shape) / math.sqrt(shape[1])
+    return w
+
+
+@pytest.mark.parametrize("gating", [False, "per-head", "per-head-hd", "elementwise"])
+def test_mhsa_equals_separately_written_glue(gating):
+    """mhsa_forward against the composition projection -> apply_rope -> caller_glue -> output projection
+    (caller_glue covers the gate only in its per-head form: the other two are applied here by hand)."""
+    b, S, H, Hkv, d = 2, 11, 4, 2, 8
+    d_model = H * d
+    w = _mhsa_weights(d_model, H, Hkv, gating, True, True)
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(b, S, d_model, generator=g, dtype=F64)
+    v1 = torch.randn(H * b, S, d, generator=g, dtype=F64)
+    out, V = orc.mhsa_forward(x, w, n_heads=H, n_kv_heads=Hkv, max_seq_len=32, qknorm=True, gating=gating, v1=v1)
+    proj = x @ w["qkv.linear.weight"].T
+    q = proj[..., : H * d].reshape(b, S, H, d).permute(0, 2, 1, 3)
+    k = proj[..., H * d : (H + Hkv) * d].reshape(b, S, Hkv, d).permute(0, 2, 1, 3)
+    v = proj[..., (H + Hkv) * d :].reshape(b, S, Hkv, d).permute(0, 2, 1, 3)
+    cos, sin = orc.rope_tables(32, 10000.0, d)
+    gl = None
+    if gating == "per-head":
+        gl = x @ w["attn_gate.linear.weight"].T
+    elif gating == "per-head-hd":
+        gl = x[..., :d] @ w["attn_gate.linear.weight"].T
+    cat, V2 = orc.caller_glue(orc.apply_rope(q, cos, sin), orc.apply_rope(k, cos, sin), v, w["sdpa_qknorm.gain"], v1=v1,
+                              alpha1=w["alpha1"], alpha2=w["alpha2"], scale=w["scale"], gate_logits=gl)
+    if gating == "elementwise":
+        cat = 2.0 * torch.sigmoid(x @ w["attn_gate.linear.weight"].T) * cat
+    assert torch.allclose(out, cat @ w["out.linear.weight"].T, atol=1e-11)
+    assert torch.allclose(V, V2, atol=1e-12)
+
+
+def test_mhsa_python_loop_without_qknorm():
+    """Per (batch, head) loops over plain softmax attention on a tiny case: catches a wrong head split of the
+    projection, a wrong GQA map or a wrong concat order."""
+    b, S, H, Hkv, d = 2, 5, 4, 2, 4
+    d_model = H * d
+    w = _mhsa_weights(d_model, H, Hkv, False, False, False)
+    x = torch.randn(b, S, d_model, generator=torch.Generator().manual_seed(8), dtype=F64)
+    out, V = orc.mhsa_forward(x, w, n_heads=H, n_kv_heads=Hkv, max_seq_len=16, qknorm=False)
+    cos, sin = orc.rope_tables(16, 10000.0, d)
+    proj = x @ w["qkv.linear.weight"].T
+    cat = torch.zeros(b, S, d_model, dtype=F64)
+    for bi in range(b):
+        for h in range(H):
+            gkv = h // (H // Hkv)
+            qh = orc.apply_rope(proj[bi, :, h * d : (h + 1) * d], cos, sin)
+            kh = orc.apply_rope(proj[bi, :, (H + gkv) * d : (H + gkv + 1) * d], cos, sin)
+            vh = proj[bi, :, (H + Hkv + gkv) * d : (H + Hkv + gkv + 1) * d]
+            for i in range(S):
+                sc = torch.stack([(qh[i] * kh[j]).sum() / math.sqrt(d) for j in range(i + 1)])
+                pr = torch.softmax(sc, 0)
+                cat[bi, i, h * d : (h + 1) * d] = sum(pr[j] * vh[j] for j in range(i + 1))
+            # with the buffers (1, 0, 1) the value-residual line only multiplies by rsqrt(1 + 1e-8)
+            assert torch.allclose(V[h * b + bi], vh * (1 + 1e-8) ** -0.5, atol=1e-12)
+    assert torch.allclose(out, (cat * (1 + 1e-8) ** -0.5) @ w["out.linear.weight"].T, atol=1e-11)
+
+
+@pytest.mark.parametrize("qknorm", [True, False])
+def test_mhsa_cached_steps_equal_one_full_pass(qknorm):
+    """Prefill + single-token steps through the KV cache reproduce the rows of one full causal pass
+    (positions and the causal diagonal both shift by the cache length, attention.py:185-198)."""
+    b, S, H, Hkv, d = 2, 9, 4, 2, 8
+    d_model = H * d
+    w = _mhsa_weights(d_model, H, Hkv, "per-head", True, qknorm)
+    x = torch.randn(b, S, d_model, generator=torch.Generator().manual_seed(10), dtype=F64)
+    kw = dict(n_heads=H, n_kv_heads=Hkv, max_seq_len=16, qknorm=qknorm, gating="per-head")
+    full, V_full = orc.mhsa_forward(x, w, **kw)
+    cache = {"keys": None, "values": None}
+    outs = [orc.mhsa_forward(x[:, :6], w, cache=cache, **kw)[0]]
+    for t in range(6, S):
+        o, V_t = orc.mhsa_forward(x[:, t : t + 1], w, cache=cache, **kw)
+        outs.append(o)
+    assert cache["keys"].shape == (H * b, S, d)
+    assert torch.allclose(torch.cat(outs, dim=1), full, atol=1e-11)
+    assert torch.allclose(V_t, V_full, atol=1e-12)

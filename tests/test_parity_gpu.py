@@ -9,8 +9,8 @@ import pytest
 import torch
 
 from oracle import qknorm_attn_oracle as orc
-from sample_efficient_gpt_amd import (CONFIGS, FlashAttnFunc, QKNormFlashAttnFunc, SelfDotProductAttnQKNorm, make_inputs,
-                                      qknorm_attention, qknorm_attention_op)
+from sample_efficient_gpt_amd import (CONFIGS, FlashAttnFunc, KVCache, MultiHeadSelfAttention, QKNormFlashAttnFunc,
+                                      SelfDotProductAttnQKNorm, make_inputs, qknorm_attention, qknorm_attention_op)
 from tests.parity_util import compare, gen, run_gpu, run_oracle, scalar_gain_scale
 
 pytestmark = pytest.mark.gpu
@@ -509,3 +509,127 @@ def test_strided_projection_views(gpu_device):
     y = qknorm_attention(q, k, v, x["g_q"].to(gpu_device), x["g_k"].to(gpu_device))
     ref = run_oracle(x, backward=False)
     compare({"y": y.cpu()}, ref, BF16, names=["y"])
+
+
+# ------------------------------------------------------------------ the whole attention module around one kernel call
+
+
+def _module_and_oracle_weights(device, dtype, d_model, H, Hkv, qknorm, value_residual, gating, seed):
+    torch.manual_seed(seed)
+    m = MultiHeadSelfAttention(d_model, H, Hkv, max_seq_len=1024, qknorm=qknorm, value_residual=value_residual, gating=gating)
+    with torch.no_grad():
+        if qknorm:
+            m.sdpa_qknorm.gain.fill_(1.3)
+        if value_residual:
+            m.alpha1.fill_(0.8); m.alpha2.fill_(0.5); m.scale.fill_(1.1)
+    for name in ("qkv", "out", "attn_gate"):
+        if hasattr(m, name):
+            getattr(m, name).to(dtype)
+    m = m.to(device)
+    w = {n: t.detach().cpu().double().requires_grad_(True) for n, t in m.state_dict().items()}
+    rope = (m.rope.cos.detach().cpu().double(), m.rope.sin.detach().cpu().double())
+    return m, w, rope
+
+
+def _weight_close(got, ref, dtype, name, yardstick=None):
+    """Weight gradients are sums over every token: tolerance relative to the largest entry (norm-wise).
+    A scalar parameter's gradient is ONE sum over every element of the layer, so the bf16 rounding noise of
+    the summands does not shrink with the (cancelling) total: for those the relative part refers to
+    `yardstick`, the sum of the magnitudes of the partial gradients the scalar is the total of (the fp32
+    cases pin the same gradients tightly)."""
+    tol = {BF16: (2e-2, 1e-2), F32: (2e-4, 2e-4)}[dtype]
+    err = (got.double() - ref).abs().max()
+    scale = ref.abs().max() if yardstick is None or dtype != BF16 else max(float(ref.abs().max()), yardstick)
+    bound = tol[0] + tol[1] * scale
+    assert err <= bound, f"{name}: max abs err {float(err):.3e} > {float(bound):.3e} (ref max {float(ref.abs().max()):.3e})"
+
+
+@pytest.mark.parametrize(
+    "dtype,H,Hkv,d,S,qknorm,value_residual,gating,use_v1",
+    [
+        (F32, 4, 2, 64, 100, True, True, "per-head", True),
+        (F32, 2, 2, 32, 70, False, False, False, False),
+        (BF16, 6, 2, 64, 256, True, True, "per-head", True),      # the IMU-1 layer shape in small
+        (BF16, 6, 2, 64, 200, True, True, "per-head", False),     # first layer: v1 is None
+        (BF16, 4, 4, 64, 130, True, False, "per-head-hd", False),
+        (BF16, 4, 1, 128, 96, False, False, "elementwise", False),
+        (BF16, 4, 2, 64, 160, True, False, False, False),
+    ],
+)
+def test_mhsa_module_matches_oracle(gpu_device, dtype, H, Hkv, d, S, qknorm, value_residual, gating, use_v1):
+    """MultiHeadSelfAttention (projection -> ONE fused kernel call -> output projection) against the oracle's
+    step-by-step restatement of attention.py:175-267 on the same weights: outputs, the value tensor handed to
+    later layers, and the gradients of x, v1 and every parameter."""
+    b, d_model = 2, H * d
+    m, w, rope = _module_and_oracle_weights(gpu_device, dtype, d_model, H, Hkv, qknorm, value_residual, gating, seed=3)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(b, S, d_model, generator=g).to(dtype)
+    d_out = torch.randn(b, S, d_model, generator=g).to(dtype)
+    v1 = torch.randn(H // Hkv * 0 + Hkv * b, S, d, generator=g).to(dtype) if use_v1 else None   # [(hkv b), S, d]
+    print(f"mhsa case {dtype} H={H} Hkv={Hkv} d={d} S={S} qknorm={qknorm} vr={value_residual} gating={gating} v1={use_v1}", flush=True)
+    # oracle (fp64 on the same bits); v1 in the reference's expanded layout
+    xr = x.double().requires_grad_(True)
+    v1r = None if v1 is None else v1.double().requires_grad_(True)
+    v1x = None if v1 is None else orc.expand_kv_flat(v1r, Hkv, H)
+    ref_out, ref_V = orc.mhsa_forward(xr, w, n_heads=H, n_kv_heads=Hkv, qknorm=qknorm, gating=gating, v1=v1x, rope=rope)
+    ref_out.backward(d_out.double())
+    # product
+    xd = x.to(gpu_device).requires_grad_(True)
+    v1d = None if v1 is None else v1.to(gpu_device).requires_grad_(True)
+    out, V = m(xd, v1=v1d)
+    assert out.shape == (b, S, d_model) and V.shape == (b, Hkv, S, d)
+    out.backward(d_out.to(gpu_device))
+    torch.cuda.synchronize()
+    tol = dict(atol=2e-2, rtol=1e-2) if dtype == BF16 else dict(atol=2e-4, rtol=2e-4)
+    assert torch.allclose(out.detach().cpu().double(), ref_out.detach(), **tol), (out.detach().cpu().double() - ref_out.detach()).abs().max()
+    ref_V_native = orc.unflatten_heads(ref_V.detach(), H)[:, :: H // Hkv]
+    assert torch.allclose(V.detach().cpu().double(), ref_V_native, **tol)
+    _weight_close(xd.grad.cpu(), xr.grad, dtype, "dx")
+    if v1 is not None:
+        _weight_close(v1d.grad.cpu(), v1r.grad, dtype, "dv1")
+    # yardsticks of the scalar parameters: the gain as a vector of equal entries gives its per-dimension
+    # gradients; alpha1 / alpha2 / scale act through (c1, c2), whose gradients are sums over (batch, kv head)
+    yard = {}
+    if dtype == BF16:
+        wv = {n: t.detach().clone().requires_grad_(True) for n, t in w.items()}
+        if qknorm:
+            wv["sdpa_qknorm.gain"] = w["sdpa_qknorm.gain"].detach().expand(d).clone().requires_grad_(True)
+        pieces = {}
+        if value_residual:  # one (alpha1, alpha2, scale) copy per flattened value row
+            for n in ("alpha1", "alpha2", "scale"):
+                pieces[n] = w[n].detach().expand(H * b, 1, 1).clone().requires_grad_(True)
+                wv[n] = pieces[n]
+        o2, _ = orc.mhsa_forward(x.double(), wv, n_heads=H, n_kv_heads=Hkv, qknorm=qknorm, gating=gating,
+                                 v1=None if v1 is None else orc.expand_kv_flat(v1.double(), Hkv, H), rope=rope)
+        o2.backward(d_out.double())
+        if qknorm:
+            yard["sdpa_qknorm.gain"] = float(wv["sdpa_qknorm.gain"].grad.abs().sum())
+        for n, t in pieces.items():
+            yard[n] = float(t.grad.abs().sum())
+        print("scalar-parameter yardsticks", yard, flush=True)
+    for n, p in m.named_parameters():
+        _weight_close(p.grad.cpu(), w[n].grad, dtype, n, yard.get(n))
+
+
+def test_mhsa_module_generation_with_cache(gpu_device):
+    """Prefill + single-token steps through KVCache (raw, un-expanded keys; split-key decode kernels under
+    no_grad) reproduce one full causal pass and the oracle's cached run."""
+    H, Hkv, d, S0, S = 6, 2, 64, 150, 154
+    b, d_model = 2, H * d
+    m, w, rope = _module_and_oracle_weights(gpu_device, BF16, d_model, H, Hkv, True, True, "per-head", seed=9)
+    x = torch.randn(b, S, d_model, generator=torch.Generator().manual_seed(12)).to(BF16)
+    xd = x.to(gpu_device)
+    with torch.no_grad():
+        full, V_full = m(xd)
+        cache = KVCache()
+        outs = [m(xd[:, :S0], kv_cache=cache)[0]]
+        for t in range(S0, S):
+            o, V_t = m(xd[:, t : t + 1], kv_cache=cache)
+            outs.append(o)
+    assert cache.length == S and cache.keys.shape == (b, Hkv, S, d)
+    steps = torch.cat(outs, dim=1)
+    assert torch.allclose(steps.float(), full.float(), atol=2e-2, rtol=1e-2)
+    assert torch.allclose(V_t.float(), V_full.float(), atol=1e-2, rtol=1e-2)
+    wd = {n: t.detach() for n, t in w.items()}
+    ref, _ = orc.mhsa_forward(x.double(), wd, n_heads=H, n_kv_heads=Hkv, qknorm=True, gating="per-head", rope=rope)
+    assert torch.allclose(steps.cpu().double(), ref, atol=2e-2, rtol=1e-2)
