@@ -13,7 +13,9 @@ from .function import _fill_common, _rope_arg
 
 class AttnPlan:
     """Binds canonical-layout tensors (q [B,H,S,D], k/v [B,Hkv,S,D], ...) once; `forward()`,
-    `backward()` and `backward_stage(i)` then only enqueue kernels on the current stream."""
+    `backward()` and `backward_stage(i)` then only enqueue kernels on the current stream.  Nothing is
+    allocated, copied or cleared per call, so a forward + backward pair can be captured into a HIP graph
+    (`torch.cuda.graph`) and replayed."""
 
     def __init__(self, x: dict, *, eps=1e-6, sm_scale=None, gate_scale=2.0, causal=True, q_start=0, backward=True,
                  rope_cos=None, rope_sin=None, rope_q_pos0=None, rope_k_pos0=0, qk_norm=True):
@@ -51,7 +53,12 @@ class AttnPlan:
             p.dg_q, p.dg_k, p.dvr_coef = _lib.ptr(self.dg_q), _lib.ptr(self.dg_k), _lib.ptr(self.dcoef)
             self.ws = _lib.alloc_workspace(self.lib, p, _lib.SEGPT_WS_BWD, dev)
             p.workspace, p.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
-        self.stream = torch.cuda.current_stream(dev).cuda_stream
+        self.dev = dev
+
+    @property
+    def stream(self):
+        """The device's current stream at call time (so that the calls can be captured into a graph)."""
+        return torch.cuda.current_stream(self.dev).cuda_stream
 
     def _chk(self, rc, what):
         if rc != 0:

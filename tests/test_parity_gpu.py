@@ -140,6 +140,54 @@ def test_cfg3_imu1_fwd_bwd_full_size(gpu_device):
     compare(run_gpu(xb, gpu_device, **kw), run_oracle(xb, **kw), c.dtype, names=["dg_q", "dg_k"], label="cfg3[b=0] ")
 
 
+def test_cfg3_full_size_exact_properties(gpu_device):
+    """Size-independent properties at the IMU-1 shape, all bit-exact: (1) scaling v or dO by a power of two
+    scales what is linear in them and leaves the rest alone; (2) causality: changing tokens >= t leaves the
+    outputs and dq of rows < t alone, changing queries / dO of rows < t leaves dk, dv of rows >= t alone;
+    (3) the batch entries are independent: reversing the batch reverses the results."""
+    c = CONFIGS[3]
+    x = make_inputs(c)
+    kw = dict(eps=c.eps, sm_scale=c.sm_scale)
+    print("cfg3 exact properties", flush=True)
+    base = run_gpu(x, gpu_device, **kw)
+    eq = lambda a, b: torch.equal(a.float(), b.float())
+    # (1a) v -> 2 v
+    got = run_gpu(dict(x, v=x["v"] * 2), gpu_device, **kw)
+    assert eq(got["y"], base["y"] * 2) and eq(got["lse"], base["lse"])
+    assert eq(got["dq"], base["dq"] * 2) and eq(got["dk"], base["dk"] * 2) and eq(got["dv"], base["dv"])
+    assert eq(got["dg_q"], base["dg_q"] * 2)
+    # (1b) dO -> dO / 4
+    got = run_gpu(dict(x, d_o=x["d_o"] * 0.25), gpu_device, **kw)
+    assert eq(got["y"], base["y"])
+    for n in ("dq", "dk", "dv", "dg_q", "dg_k"):
+        assert eq(got[n], base[n] * 0.25), n
+    # (2a) new q, k, v, dO from token t on
+    t = 1111
+    g = torch.Generator().manual_seed(77)
+    xp = dict(x)
+    for n in ("q", "k", "v", "d_o"):
+        xp[n] = x[n].clone()
+        xp[n][:, :, t:] = torch.randn(x[n][:, :, t:].shape, generator=g).to(x[n].dtype)
+    got = run_gpu(xp, gpu_device, **kw)
+    for n in ("y", "lse", "dq"):
+        assert eq(got[n][:, :, :t], base[n][:, :, :t]), n
+        assert not eq(got[n][:, :, t:], base[n][:, :, t:]), n
+    # (2b) new q, dO before token t
+    xp = dict(x)
+    for n in ("q", "d_o"):
+        xp[n] = x[n].clone()
+        xp[n][:, :, :t] = torch.randn(x[n][:, :, :t].shape, generator=g).to(x[n].dtype)
+    got = run_gpu(xp, gpu_device, **kw)
+    for n in ("dk", "dv"):
+        assert eq(got[n][:, :, t:], base[n][:, :, t:]), n
+        assert not eq(got[n][:, :, :t], base[n][:, :, :t]), n
+    # (3) reversed batch
+    got = run_gpu({n: (v.flip(0) if n in ("q", "k", "v", "d_o") else v) for n, v in x.items()}, gpu_device, **kw)
+    for n in ("y", "lse", "dq", "dk", "dv"):
+        assert eq(got[n].flip(0), base[n]), n
+    assert torch.allclose(got["dg_q"], base["dg_q"], atol=2e-2, rtol=1e-2)
+
+
 def test_cfg4_long_context_extras_full_size(gpu_device):
     _slice_check(gpu_device, CONFIGS[4], [(1, 3)], odtype=torch.float32)
 
@@ -633,3 +681,42 @@ def test_mhsa_module_generation_with_cache(gpu_device):
     wd = {n: t.detach() for n, t in w.items()}
     ref, _ = orc.mhsa_forward(x.double(), wd, n_heads=H, n_kv_heads=Hkv, qknorm=True, gating="per-head", rope=rope)
     assert torch.allclose(steps.cpu().double(), ref, atol=2e-2, rtol=1e-2)
+
+
+# ------------------------------------------------------------------ HIP graph capture of a forward + backward pair
+
+
+def test_graph_replays_match_eager_step(gpu_device):
+    """A captured forward + backward (the library allocates, copies and clears nothing per call) replayed
+    several times, with eager work and new inputs between the replays: every replay is bit-identical to the
+    eager step on the same inputs."""
+    from sample_efficient_gpt_amd.plan import AttnPlan
+
+    c = CONFIGS[4].scaled(B=1, S=640)  # gate + value residual: every kernel and the reduce stage take part
+    x = make_inputs(c, device=gpu_device)
+    plan = AttnPlan(x, eps=c.eps, sm_scale=c.sm_scale, gate_scale=c.gate_scale)
+    outs = [plan.y, plan.lse, plan.dq, plan.dk, plan.dv, plan.dv_first, plan.dgate, plan.dg_q, plan.dg_k, plan.dcoef]
+
+    def eager():
+        plan.forward()
+        plan.backward(kv_prepared=True)
+        torch.cuda.synchronize()
+        return [t.clone() for t in outs]
+
+    ref0 = eager()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.forward()
+        plan.backward(kv_prepared=True)
+    gen_ = torch.Generator(device=gpu_device).manual_seed(5)
+    for it in range(4):
+        if it:  # new inputs in the bound buffers (eager kernels between the replays)
+            for n in ("q", "k", "v", "d_o"):
+                x[n].copy_(torch.randn(x[n].shape, generator=gen_, device=gpu_device).to(x[n].dtype))
+        ref = eager() if it else ref0
+        for t in outs:
+            t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, ref):
+            assert torch.equal(a, b), f"replay {it} differs from the eager step"
