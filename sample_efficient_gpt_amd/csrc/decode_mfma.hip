@@ -49,9 +49,12 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(KArgs a) {
   constexpr int MB = D / 32;
   constexpr int RS = DecTile<D>::kRS;
   const segpt_attn_params& p = a.p;
-  __shared__ __attribute__((aligned(16))) uint16_t vt[4][32 * RS];  // wave-private V' tiles
+  // wave-private V' tiles during the key loop; afterwards the same memory holds the per-wave O^T partials
+  constexpr int kVtBytes = 4 * 32 * RS * 2, kOsmBytes = 4 * D * 32 * 4;
+  __shared__ __attribute__((aligned(16))) char tile_mem[kVtBytes > kOsmBytes ? kVtBytes : kOsmBytes];
+  uint16_t (*vt)[32 * RS] = reinterpret_cast<uint16_t (*)[32 * RS]>(tile_mem);
+  float (*osm)[D][32] = reinterpret_cast<float (*)[D][32]>(tile_mem);
   __shared__ __attribute__((aligned(16))) float gsm[D];
-  __shared__ __attribute__((aligned(16))) float osm[4][D][32];      // per-wave O^T partials for the merge
   __shared__ float msm[4][32], lsm[4][32];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -195,6 +198,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(KArgs a) {
   }
 
   // ---- merge the four waves (different keys, same queries) and write this split's partial
+  __syncthreads();  // every wave is done with its V' tile: the memory is reused for the partials
   const float l_tot = half_sum(l_run);
   if (hh == 0) { msm[wave][ln] = m_run; lsm[wave][ln] = l_tot; }
 #pragma unroll
@@ -219,75 +223,87 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(KArgs a) {
 }
 
 // One workgroup per (batch, kv head, query row): merges the splits, normalises, gates, writes y (bf16) and lse
-// (natural log).  Thread d owns output column d; the split weights 2^(M_s - M) are shared through LDS.
-constexpr int kMergeThreads = 128;
+// (natural log).  Thread (group gi, column d) sums the splits gi, gi + G, ... of output column d (G = threads / D);
+// its first partial values are requested before the split statistics are reduced, so that the kernel is about
+// two memory round trips long whatever the number of splits.  Every sum has a fixed order: deterministic.
+constexpr int kMergeThreads = 256;
 constexpr int kMaxSplits = 512;
+constexpr int kMergeEarly = 16;  // partial values per thread requested up front
 
 __global__ __launch_bounds__(kMergeThreads) void decode_merge_kernel(KArgs a) {
   const segpt_attn_params& p = a.p;
   __shared__ float wsm[kMaxSplits];
-  __shared__ float red[kMergeThreads];
-  const int D = p.D, tid = threadIdx.x;
+  __shared__ float redm[4], redl[4];
+  __shared__ float part[kMergeThreads];
+  const int D = p.D, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rep = p.H / p.Hkv;
   const int n_rows = rep * p.Sq;
   const int n = blockIdx.x % n_rows, bg = blockIdx.x / n_rows;
   const int g = bg % p.Hkv, b = bg / p.Hkv;
   const int S = a.dec_splits;
-  const float* so = a.dec_part + (int64_t)bg * S * 32 * D;
+  const int G = kMergeThreads / D, gi = tid / D, d = tid - gi * D;
+  const float* col = a.dec_part + (int64_t)bg * S * 32 * D + (int64_t)n * D + d;
   const float* ss = a.dec_stat + (int64_t)bg * S * 32 * 2;
+  float pv[kMergeEarly];
+#pragma unroll
+  for (int u = 0; u < kMergeEarly; ++u) {
+    const int sp = gi + G * u;
+    pv[u] = sp < S ? col[(int64_t)sp * 32 * D] : 0.f;
+  }
   float m = -INFINITY;
-  for (int s = tid; s < S; s += kMergeThreads) m = fmaxf(m, ss[(s * 32 + n) * 2]);
-  red[tid] = m;
+  for (int sp = tid; sp < S; sp += kMergeThreads) m = fmaxf(m, ss[(sp * 32 + n) * 2]);
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if (lane == 0) redm[wave] = m;
   __syncthreads();
-  for (int o = kMergeThreads / 2; o > 0; o >>= 1) {
-    if (tid < o) red[tid] = fmaxf(red[tid], red[tid + o]);
-    __syncthreads();
-  }
-  const float M = red[0];
-  __syncthreads();
+  const float M = fmaxf(fmaxf(redm[0], redm[1]), fmaxf(redm[2], redm[3]));
   float l = 0.f;
-  for (int s = tid; s < S; s += kMergeThreads) {
-    const float w = exp2f(ss[(s * 32 + n) * 2] - M);
-    wsm[s] = w;
-    l += ss[(s * 32 + n) * 2 + 1] * w;
+  for (int sp = tid; sp < S; sp += kMergeThreads) {
+    const float w = exp2f(ss[(sp * 32 + n) * 2] - M);  // a split with nothing visible has (-inf, 0): weight 0
+    wsm[sp] = w;
+    l += ss[(sp * 32 + n) * 2 + 1] * w;
   }
-  red[tid] = l;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) l += __shfl_xor(l, o, 64);
+  if (lane == 0) redl[wave] = l;
+  __syncthreads();  // also publishes wsm
+  const float L = (redl[0] + redl[1]) + (redl[2] + redl[3]);
+  float acc = 0.f;
+#pragma unroll
+  for (int u = 0; u < kMergeEarly; ++u) {
+    const int sp = gi + G * u;
+    if (sp < S) acc += pv[u] * wsm[sp];
+  }
+  for (int sp = gi + G * kMergeEarly; sp < S; sp += G) acc += col[(int64_t)sp * 32 * D] * wsm[sp];
+  part[tid] = acc;
   __syncthreads();
-  for (int o = kMergeThreads / 2; o > 0; o >>= 1) {  // fixed tree: deterministic
-    if (tid < o) red[tid] += red[tid + o];
-    __syncthreads();
-  }
-  const float L = red[0];
   const int hq = n / p.Sq, qi = n % p.Sq;
   const int h = g * rep + hq;
-  float f = 1.0f / L;
-  if (p.gate.ptr) {
-    const float z = bf16_to_f32(reinterpret_cast<const uint16_t*>(p.gate.ptr)[(int64_t)b * p.gate.stride_b + (int64_t)qi * p.gate.stride_s + (int64_t)h * p.gate.stride_h]);
-    f *= p.gate_scale / (1.0f + __expf(-z));
-  }
   if (tid == 0) p.lse[((int64_t)b * p.H + h) * p.Sq + qi] = (M + log2f(L)) * kLn2;
   if (tid < D) {
-    const float* col = so + (int64_t)n * D + tid;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    int s = 0;
-    for (; s + 3 < S; s += 4) {
-#pragma unroll
-      for (int u = 0; u < 4; ++u) acc[u] += col[(int64_t)(s + u) * 32 * D] * wsm[s + u];
+    float f = 1.0f / L;
+    if (p.gate.ptr) {
+      const float z = bf16_to_f32(reinterpret_cast<const uint16_t*>(p.gate.ptr)[(int64_t)b * p.gate.stride_b + (int64_t)qi * p.gate.stride_s + (int64_t)h * p.gate.stride_h]);
+      f *= p.gate_scale / (1.0f + __expf(-z));
     }
-    for (; s < S; ++s) acc[0] += col[(int64_t)s * 32 * D] * wsm[s];
-    row_ptr_mut<uint16_t>(p.o, b, h, qi)[tid] = f32_to_bf16(((acc[0] + acc[1]) + (acc[2] + acc[3])) * f);
+    float tot = part[tid];
+    for (int x = 1; x < G; ++x) tot += part[x * D + tid];
+    row_ptr_mut<uint16_t>(p.o, b, h, qi)[tid] = f32_to_bf16(tot * f);
   }
 }
 
 }  // namespace
 
 // Split plan of a decode-shaped call: keys [0, kend) in `splits` chunks of `chunk` keys (a multiple of 128):
-// enough workgroups for about two per CU, no empty split.  Returns the scratch bytes the partials need.
+// enough workgroups for one resident round, no empty split: three per CU at head_dim 64 (what the kernel's
+// registers allow; measured 17 % faster than two per CU, four is slower again), one per CU at head_dim 128
+// (15 % faster than two).  Returns the scratch bytes the partials need.
 size_t decode_plan(const segpt_attn_params& p, int* kend_out, int* splits_out, int* chunk_out) {
   int kend = p.Sk;
   if (p.causal && p.Sq + p.q_start < kend) kend = p.Sq + p.q_start;
   const int groups = p.B * p.Hkv;
-  int s = (512 + groups - 1) / groups;
+  const int target = p.D == 64 ? 768 : 256;
+  int s = (target + groups - 1) / groups;
   const int max_s = (kend + kDecKeysPerStep - 1) / kDecKeysPerStep;
   if (s > max_s) s = max_s;
   if (s > kMaxSplits) s = kMaxSplits;
