@@ -94,9 +94,20 @@ def scalar_gain_scale(x, **kw):
     return {"dg_q": float(ref["dg_q"].abs().sum())}
 
 
-def compare(got, ref, dtype, names=None, label="", scales=None):
+def value_residual_scale(x, ref):
+    """Yardstick for the gradients of the two value-residual coefficients: dc1 = sum(dV' * v), dc2 = sum(dV' * v_first)
+    over every key row and column; their bf16 rounding errors add up, so the relative tolerance refers to the
+    sum of the magnitudes of the summands (dV' = dv / c1 from the oracle) instead of the cancelled total."""
+    c1 = float(x["vr_coef"][0])
+    dvm = ref["dv"].double() / c1
+    return {"dvr_coef": float(max((dvm * x["v"].double()).abs().sum(), (dvm * x["v_first"].double()).abs().sum()))}
+
+
+def compare(got, ref, dtype, names=None, label="", scales=None, outliers=None):
     """Asserts |got - ref| <= atol + rtol*|ref| for every output; returns {name: max_abs_err}.
-    `scales` overrides the magnitude the relative part refers to for the named outputs."""
+    `scales` overrides the magnitude the relative part refers to for the named outputs.
+    `outliers` = (fraction, factor): that fraction of a tensor's elements may exceed the bound, by at most
+    `factor` (None: no element may)."""
     tol = TOL[dtype]
     errs = {}
     failures = []
@@ -113,6 +124,8 @@ def compare(got, ref, dtype, names=None, label="", scales=None):
         bound = tol["atol"] + tol["rtol"] * scale
         errs[n] = float(err.max())
         bad = err > bound
+        if outliers is not None and bad.any() and int(bad.sum()) <= outliers[0] * bad.numel() and not (err > outliers[1] * bound).any():
+            bad = bad & False
         if bad.any():
             failures.append(f"{label}{n}: {int(bad.sum())}/{bad.numel()} outside tolerance, max abs err {errs[n]:.3e} "
                             f"(ref max {float(r.abs().max()):.3e})")
