@@ -55,6 +55,7 @@ def test_cfg1_fp32_forward(gpu_device):
         (1, 3, 3, 40, 104, 64, {"q_start": 64}, {"extras": True}),
         (1, 2, 1, 64, 64, 64, {"eps": 1e-8 / 64, "sm_scale": 1 / 64}, {"scalar_gain": True, "no_gk": True}),
         (1, 4, 2, 200, 200, 64, {"gate_scale": 2.0}, {"extras": True, "scalar_gain": True}),  # scalar q gain + vector k scale
+        (1, 2, 1, 200, 130, 64, {}, {}),   # causal with more queries than keys: rows >= 130 see every key
     ],
 )
 def test_fp32_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
@@ -82,6 +83,8 @@ def test_fp32_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
         (1, 2, 1, 1, 257, 64, {"q_start": 256}, {}),   # decode step: one query against a 257-key cache
         (8, 2, 1, 128, 128, 64, {}, {}),              # B*Hkv multiple of 8: XCD-pinned workgroup order
         (1, 2, 2, 128, 128, 64, {"eps": 1e-8 / 64, "sm_scale": 1 / 64}, {"scalar_gain": True, "no_gk": True}),
+        (2, 4, 2, 300, 130, 64, {}, {}),               # causal with more queries than keys: rows >= 130 see every key
+        (1, 2, 1, 257, 64, 128, {}, {"extras": True}),
     ],
 )
 def test_bf16_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
