@@ -229,3 +229,46 @@ def test_library_op_is_registered_with_a_shape_only_implementation():
                                                None, dev(1, 2, 70, 128), dev(2, dt=torch.float32), dev(1, 50, 4), 2.0, 1e-6, 0.1, True, 20, None, None, -1, 0, True)
         assert out[0].shape == (1, 4, 50, 128) and out[1].shape == (1, 4, 50)
         assert out[2].numel() == 2 * (2 * 70 * 128 * 2 + 255) // 256 * 256 or out[2].numel() >= 2 * 2 * 70 * 128 * 2
+
+
+def test_plain_c_program_uses_the_library(tmp_path):
+    """The boundary is a C ABI: a C99 program (gcc, no HIP or torch headers) includes the header, links the
+    shared library and calls the entry points that need no GPU; its view of the struct matches the binding's."""
+    import shutil
+    import subprocess
+
+    from sample_efficient_gpt_amd import _lib
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("gcc not found")
+    lib_path = _lib.LIB_PATH if hasattr(_lib, "LIB_PATH") else os.path.join(os.path.dirname(_lib.__file__), "libsegpt_attn.so")
+    src = tmp_path / "t.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "segpt_attn.h"
+int main(void) {
+  segpt_attn_params p;
+  memset(&p, 0, sizeof p);
+  p.struct_bytes = (int)sizeof p;
+  p.dtype = SEGPT_DTYPE_BF16; p.B = 2; p.H = 6; p.Hkv = 2; p.Sq = 100; p.Sk = 100; p.D = 64;
+  printf("%d %zu %zu %zu %d %s\n", segpt_abi_version(), sizeof p, segpt_attn_workspace_bytes(&p, SEGPT_WS_KV),
+         segpt_attn_workspace_bytes(&p, SEGPT_WS_BWD), segpt_attn_fwd(&p, NULL), segpt_strerror(SEGPT_E_HEAD_DIM));
+  return 0;
+}
+''')
+    exe = tmp_path / "t"
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(_lib.__file__))), "include")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{inc}", str(src), "-o", str(exe), lib_path,
+                    f"-Wl,-rpath,{os.path.dirname(lib_path)}", "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    out = subprocess.run([str(exe)], check=True, stdout=subprocess.PIPE, text=True).stdout.split(maxsplit=5)
+    lib = _lib.load()
+    p = _lib.new_params()
+    p.dtype, p.B, p.H, p.Hkv, p.Sq, p.Sk, p.D = _lib.SEGPT_DTYPE_BF16, 2, 6, 2, 100, 100, 64
+    assert int(out[0]) == lib.segpt_abi_version()
+    assert int(out[1]) == C.sizeof(p)
+    assert int(out[2]) == lib.segpt_attn_workspace_bytes(p, _lib.SEGPT_WS_KV) == (2 * 2 * 100 * 64 * 2 + 255) // 256 * 256
+    assert int(out[3]) == lib.segpt_attn_workspace_bytes(p, _lib.SEGPT_WS_BWD)
+    assert int(out[4]) < 0  # argument error (no tensors bound), reported before any launch
+    assert "head_dim" in out[5]
