@@ -111,7 +111,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(KArgs a) {
   f32x16 oacc[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) oacc[mb] = splat16(0.f);
-  float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's half of the keys
+  float m_run = -INFINITY, l_run[2] = {0.f, 0.f};  // l_run: this lane's half of the keys, as two partial sums
 
   // keys [k_lo, k_hi) of this split; wave w takes the 32-key blocks w, w+4, ...
   const int k_lo = split * a.dec_chunk;
@@ -179,7 +179,8 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(KArgs a) {
     const float m_use = m_new == -INFINITY ? 0.f : m_new;  // nothing visible yet: keep exp2 away from inf - inf
     const float corr = fast_exp2(m_run - m_use);           // m_run = -inf gives 0
     m_run = m_new;
-    l_run *= corr;
+    l_run[0] *= corr;
+    l_run[1] *= corr;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -199,7 +200,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(KArgs a) {
 
   // ---- merge the four waves (different keys, same queries) and write this split's partial
   __syncthreads();  // every wave is done with its V' tile: the memory is reused for the partials
-  const float l_tot = half_sum(l_run);
+  const float l_tot = half_sum(l_run[0] + l_run[1]);
   if (hh == 0) { msm[wave][ln] = m_run; lsm[wave][ln] = l_tot; }
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)

@@ -139,12 +139,12 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
     for (int nb = 0; nb < NQB; ++nb) oacc[mb][nb] = splat16(0.f);
   // m_ref: the value subtracted from the logits before exp2 (0 on the bounded path); l_run: this lane's
   // share of the row sum (its half of the keys; halves are added in the epilogue)
-  float m_ref[NQB], l_run[NQB];
+  float m_ref[NQB], l_run[NQB][2];
   int qlim[NQB];  // last visible key of this lane's query in block nb
 #pragma unroll
   for (int nb = 0; nb < NQB; ++nb) {
     m_ref[nb] = bounded ? 0.f : -INFINITY;
-    l_run[nb] = 0.f;
+    l_run[nb][0] = l_run[nb][1] = 0.f;
     qlim[nb] = p.causal ? min(qw0 + 32 * nb + ln + p.q_start, p.Sk - 1) : p.Sk - 1;
   }
 
@@ -200,7 +200,8 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
           const float m_new = need ? mx : m_ref[nb];
           const float corr = fast_exp2(m_ref[nb] - m_new);
           m_ref[nb] = m_new;
-          l_run[nb] *= corr;
+          l_run[nb][0] *= corr;
+          l_run[nb][1] *= corr;
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -278,7 +279,7 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
   for (int nb = 0; nb < NQB; ++nb) {
     const int row = qw0 + 32 * nb + ln;
     const bool live = row < p.Sq;
-    const float l = half_sum(l_run[nb]);
+    const float l = half_sum(l_run[nb][0] + l_run[nb][1]);
     float f = fast_rcp(l);
     if (p.gate.ptr) {
       const int rc = live ? row : p.Sq - 1;

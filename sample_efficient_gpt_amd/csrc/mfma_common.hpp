@@ -191,12 +191,17 @@ __device__ __forceinline__ bf16x8 pack_c_half(const f32x16& c, int s) {
 
 // same, and adds the eight packed values to `sum` (the scalar words are summed before the vector is
 // assembled: summing elements extracted back out of the assembled vector was miscompiled by hipcc 7.2)
-__device__ __forceinline__ bf16x8 pack_c_half_sum(const f32x16& c, int s, float& sum) {
+// Two running sums (the caller adds them at the end): ONE accumulator makes every block a chain of eight dependent
+// dot instructions whose latency, not their count, is what costs (measured on a register-only skeleton of the
+// forward block: 51 % of the MFMA rate with one chain, 62 % with two or four, 63 % with no row sum at all; in
+// the forward kernel itself the scheduler already parks the sums behind the tile wait, so its time is unchanged).
+__device__ __forceinline__ bf16x8 pack_c_half_sum(const f32x16& c, int s, float (&sum)[2]) {
   const uint32_t w0 = pack_bf16x2(c[8 * s + 0], c[8 * s + 1]);
   const uint32_t w1 = pack_bf16x2(c[8 * s + 2], c[8 * s + 3]);
   const uint32_t w2 = pack_bf16x2(c[8 * s + 4], c[8 * s + 5]);
   const uint32_t w3 = pack_bf16x2(c[8 * s + 6], c[8 * s + 7]);
-  sum = add_bf16_pair(w3, add_bf16_pair(w2, add_bf16_pair(w1, add_bf16_pair(w0, sum))));
+  sum[0] = add_bf16_pair(w1, add_bf16_pair(w0, sum[0]));
+  sum[1] = add_bf16_pair(w3, add_bf16_pair(w2, sum[1]));
   const u32x4 w = {w0, w1, w2, w3};
   return as_bf16x8(w);
 }
