@@ -140,7 +140,8 @@ class MultiHeadSelfAttention(nn.Module):
             self.attn_gate = _Linear(gate_in, gate_out, device=device, dtype=dtype)
 
     def forward(self, x, token_positions=None, v1=None, kv_cache: KVCache | None = None):
-        from .function import _canon, qknorm_attention
+        from .function import _canon
+        from .library_op import qknorm_attention_op
 
         b, S, d_model = x.shape
         H, Hkv = self.n_heads, self.n_kv_heads
@@ -177,7 +178,8 @@ class MultiHeadSelfAttention(nn.Module):
         elif self.gating == "per-head-hd":
             gate_logits = self.attn_gate(x[..., :d])
         gain = self.sdpa_qknorm.gain if self.qknorm else self._unit_gain
-        y = qknorm_attention(q, k, v, gain, None, v_first=v_first, vr_coef=vr_coef, gate_logits=gate_logits, gate_scale=2.0,
+        # the registered op: one opaque node under torch.compile and non-reentrant checkpointing
+        y = qknorm_attention_op(q, k, v, gain, None, v_first=v_first, vr_coef=vr_coef, gate_logits=gate_logits, gate_scale=2.0,
                              causal=True, q_start=q_start, rope_cos=self.rope.cos, rope_sin=self.rope.sin,
                              rope_q_pos0=q_start, rope_k_pos0=0, qk_norm=self.qknorm, out_bshd=True)
         attn_cat = y.permute(0, 2, 1, 3).reshape(b, S, H * d)  # a view: the kernel wrote this layout

@@ -226,7 +226,7 @@ def test_library_op_is_registered_with_a_shape_only_implementation():
     with FakeTensorMode():  # what torch.compile sees: device tensors without storage
         dev = lambda *s, dt=torch.bfloat16: torch.empty(*s, dtype=dt, device="cuda")
         out = torch.ops.segpt.qknorm_attention(dev(1, 4, 50, 128), dev(1, 2, 70, 128), dev(1, 2, 70, 128), dev(1, dt=torch.float32),
-                                               None, dev(1, 2, 70, 128), dev(2, dt=torch.float32), dev(1, 50, 4), 2.0, 1e-6, 0.1, True, 20, None, None, -1, 0, True)
+                                               None, dev(1, 2, 70, 128), dev(2, dt=torch.float32), dev(1, 50, 4), 2.0, 1e-6, 0.1, True, 20, None, None, -1, 0, True, False)
         assert out[0].shape == (1, 4, 50, 128) and out[1].shape == (1, 4, 50)
         assert out[2].numel() == 2 * (2 * 70 * 128 * 2 + 255) // 256 * 256 or out[2].numel() >= 2 * 2 * 70 * 128 * 2
 

@@ -299,8 +299,18 @@ def test_library_op_compiled_and_checkpointed_matches_eager(gpu_device):
         for a, b in zip(ref, other):
             assert torch.equal(a, b)
     torch.library.opcheck(torch.ops.segpt.qknorm_attention,
-                          tuple(x[n].to(gpu_device) for n in names) + (2.0, 1e-6, 0.125, True, 0, None, None, -1, 0, True),
+                          tuple(x[n].to(gpu_device) for n in names) + (2.0, 1e-6, 0.125, True, 0, None, None, -1, 0, True, False),
                           test_utils=("test_schema", "test_faketensor"))
+    # every optional operand absent: the backward op then returns several empty placeholders, which must be
+    # distinct tensors (returns of a custom op may not alias one another)
+    def run_min(fn):
+        t = {n: x[n].to(gpu_device).requires_grad_(True) for n in ("q", "k", "v", "g_q")}
+        y = fn(t["q"], t["k"], t["v"], t["g_q"], None)
+        y.backward(x["d_o"].to(gpu_device))
+        return [y.detach()] + [t[n].grad for n in ("q", "k", "v", "g_q")]
+
+    for a, b in zip(run_min(qknorm_attention), run_min(qknorm_attention_op)):
+        assert torch.equal(a, b)
 
 
 # ------------------------------------------------------------------ rotary embedding fused into the loads
@@ -771,3 +781,35 @@ def test_seeded_sweep(gpu_device, case):
     if use_rope:
         kw = dict(kw, rope=orc.rope_tables(Sk + Sq + 8, 10000.0, D))
     _case(gpu_device, dtype, B, H, Hkv, Sq, Sk, D, backward=backward, seed=500 + i, gen_kw=gen_kw, outliers=(1e-4, 2.0), **kw)
+
+
+def test_mhsa_module_compiles_to_one_graph(gpu_device):
+    """torch.compile(fullgraph=True) traces the whole module (projection, the registered attention op as one
+    opaque node, gate / output projection) without a graph break; outputs and every gradient equal the eager
+    module's bit for bit.  Also under non-reentrant checkpointing, as the reference wraps its layers
+    (transformer.py:123-132)."""
+    from torch.utils.checkpoint import checkpoint
+
+    H, Hkv, d, S, b = 6, 2, 64, 192, 2
+    m, _, _ = _module_and_oracle_weights(gpu_device, BF16, H * d, H, Hkv, True, True, "per-head", seed=13)
+    g = torch.Generator().manual_seed(14)
+    x = torch.randn(b, S, H * d, generator=g).to(BF16).to(gpu_device)
+    v1 = torch.randn(Hkv * b, S, d, generator=g).to(BF16).to(gpu_device)
+    d_out = torch.randn(b, S, H * d, generator=g).to(BF16).to(gpu_device)
+
+    def run(fn):
+        m.zero_grad(set_to_none=True)
+        xi, vi = x.clone().requires_grad_(True), v1.clone().requires_grad_(True)
+        out, V = fn(xi, vi)
+        out.backward(d_out)
+        return [out.detach(), V.detach(), xi.grad, vi.grad] + [p.grad.clone() for p in m.parameters()]
+
+    print("module: eager / compiled / checkpointed", flush=True)
+    ref = run(lambda a, c: m(a, v1=c))
+    mc = torch.compile(m, backend="aot_eager", fullgraph=True)
+    compiled = run(lambda a, c: mc(a, v1=c))
+    ckpt = run(lambda a, c: checkpoint(lambda a_, c_: m(a_, v1=c_), a, c, use_reentrant=False))
+    torch.cuda.synchronize()
+    for other in (compiled, ckpt):
+        for r, o in zip(ref, other):
+            assert torch.equal(r, o)
