@@ -813,3 +813,31 @@ def test_mhsa_module_compiles_to_one_graph(gpu_device):
     for other in (compiled, ckpt):
         for r, o in zip(ref, other):
             assert torch.equal(r, o)
+
+
+def test_dropin_with_every_trailing_positional_equals_canonical_call(gpu_device):
+    """The flattened drop-in with k_gain, v_first, vr_coef, gate_logits, gate_scale, n_kv_heads, eps, sm_scale and
+    the rope tables against the canonical-layout call on the same data: same kernels, so outputs and every
+    gradient (in the order of the positionals) agree bit for bit."""
+    B, H, Hkv, S, D = 2, 6, 2, 200, 64
+    x = gen(B, H, Hkv, S, S, D, BF16, extras=True, seed=31)
+    d = gpu_device
+    cos, sin = (t.float().to(d) for t in orc.rope_tables(S, 10000.0, D))
+    names = ["q", "k", "v", "g_q", "g_k", "v_first", "vr_coef", "gate_logits"]
+    t = {n: x[n].to(d).requires_grad_(True) for n in names}
+    y = qknorm_attention(t["q"], t["k"], t["v"], t["g_q"], t["g_k"], v_first=t["v_first"], vr_coef=t["vr_coef"],
+                         gate_logits=t["gate_logits"], gate_scale=2.0, eps=1e-5, sm_scale=0.11, rope_cos=cos, rope_sin=sin)
+    y.backward(x["d_o"].to(d))
+    flat = lambda a, h: orc.flatten_heads(a).contiguous()
+    f = {"Q": flat(x["q"], H), "K": flat(x["k"], Hkv), "V": flat(x["v"], Hkv), "VF": flat(x["v_first"], Hkv)}
+    f = {n: a.to(d).requires_grad_(True) for n, a in f.items()}
+    p = {n: x[n].to(d).requires_grad_(True) for n in ("g_q", "g_k", "vr_coef", "gate_logits")}
+    O = QKNormFlashAttnFunc.apply(f["Q"], f["K"], f["V"], p["g_q"], True, 0, p["g_k"], f["VF"], p["vr_coef"], p["gate_logits"],
+                                  2.0, Hkv, 1e-5, 0.11, cos, sin)
+    O.backward(flat(x["d_o"], H).to(d))
+    torch.cuda.synchronize()
+    assert torch.equal(O, flat(y.detach(), H))
+    assert torch.equal(f["Q"].grad, flat(t["q"].grad, H)) and torch.equal(f["K"].grad, flat(t["k"].grad, Hkv))
+    assert torch.equal(f["V"].grad, flat(t["v"].grad, Hkv)) and torch.equal(f["VF"].grad, flat(t["v_first"].grad, Hkv))
+    for n in ("g_q", "g_k", "vr_coef", "gate_logits"):
+        assert torch.equal(p[n].grad, t[n].grad), n
