@@ -102,7 +102,8 @@ def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scal
     kv_ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_KV, q.device)
     p.kv_workspace, p.kv_workspace_bytes = kv_ws.data_ptr(), kv_ws.numel()
     p.flags = flags | (_lib.SEGPT_FLAG_DECODE if inference else 0)
-    rc = lib.segpt_attn_fwd(p, torch.cuda.current_stream(q.device).cuda_stream)
+    with torch.cuda.device(q.device):  # the launch goes to the tensors' device, whatever the current one is
+        rc = lib.segpt_attn_fwd(p, torch.cuda.current_stream(q.device).cuda_stream)
     if rc != 0:
         raise _lib.SegptError(rc, "segpt_attn_fwd")
     return lse, kv_ws
@@ -131,7 +132,8 @@ def _backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_sca
     else:
         p.flags |= _lib.SEGPT_FLAG_KV_PREPARED
     p.kv_workspace, p.kv_workspace_bytes = kv_ws.data_ptr(), kv_ws.numel()
-    rc = lib.segpt_attn_bwd(p, torch.cuda.current_stream(dev).cuda_stream)
+    with torch.cuda.device(dev):
+        rc = lib.segpt_attn_bwd(p, torch.cuda.current_stream(dev).cuda_stream)
     if rc != 0:
         raise _lib.SegptError(rc, "segpt_attn_bwd")
     return dg_q, dg_k, dcoef
