@@ -184,11 +184,11 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   auto step = [&](auto masked_c, uint32_t tr, int kb, int jb, uint32_t next_rm, int next_kb) {
     constexpr bool MASKED = decltype(masked_c)::value != 0;
     f32x16 s = c_lse, dpv = c_del;
+    // the S chain first, then the dP chain: exp2 of the finished scores runs behind the dP MFMAs
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      s = mfma32(kf[ks], qreg[ks], s);
-      dpv = mfma32(vf[ks], doreg[ks], dpv);
-    }
+    for (int ks = 0; ks < KS; ++ks) s = mfma32(kf[ks], qreg[ks], s);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) dpv = mfma32(vf[ks], doreg[ks], dpv);
     bf16x8 kT[MB][2];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -417,10 +417,9 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
       dpv[4 * c] = d4[0]; dpv[4 * c + 1] = d4[1]; dpv[4 * c + 2] = d4[2]; dpv[4 * c + 3] = d4[3];
     }
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      s = mfma32(qf[ks], kreg[ks], s);
-      dpv = mfma32(df[ks], vreg[ks], dpv);
-    }
+    for (int ks = 0; ks < KS; ++ks) s = mfma32(qf[ks], kreg[ks], s);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) dpv = mfma32(df[ks], vreg[ks], dpv);
     bf16x8 dT[MB][2], qT[MB][2];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {

@@ -167,10 +167,12 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
     f32x16 s[NQB];
 #pragma unroll
     for (int nb = 0; nb < NQB; ++nb) s[nb] = splat16(0.f);
+    // one query block's chain after the other (not interleaved): the first block's scores are complete while
+    // the second block's MFMAs still run, so its exp2 work has something to hide behind
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
+    for (int nb = 0; nb < NQB; ++nb)
 #pragma unroll
-      for (int nb = 0; nb < NQB; ++nb) s[nb] = mfma32(kf[ks], qreg[nb][ks], s[nb]);
+      for (int ks = 0; ks < KS; ++ks) s[nb] = mfma32(kf[ks], qreg[nb][ks], s[nb]);
     bf16x8 vT[MB][2];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -221,11 +223,11 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
     }
     request_rowmajor(next_rm, next_kb);  // unconditional: past the last block the fragments are simply unused
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2)
+    for (int nb = 0; nb < NQB; ++nb)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
+      for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) oacc[mb][nb] = mfma32(vT[mb][s2], pb[s2][nb], oacc[mb][nb]);
+        for (int mb = 0; mb < MB; ++mb) oacc[mb][nb] = mfma32(vT[mb][s2], pb[s2][nb], oacc[mb][nb]);
   };
 
   // leading blocks of this wave that need no mask: every key of the block is visible to every query of the
