@@ -156,7 +156,16 @@ def test_cfg3_full_size_exact_properties(gpu_device):
     kw = dict(eps=c.eps, sm_scale=c.sm_scale)
     print("cfg3 exact properties", flush=True)
     base = run_gpu(x, gpu_device, **kw)
-    eq = lambda a, b: torch.equal(a.float(), b.float())
+
+    def eq(a, b):
+        a, b = a.float(), b.float()
+        if torch.equal(a, b):
+            return True
+        idx = (a != b).nonzero()  # say where, before the assertion fires
+        print(f"  mismatch: {idx.shape[0]} of {a.numel()} elements, first {idx[0].tolist()} last {idx[-1].tolist()}, "
+              f"max |diff| {float((a - b).abs().max()):.3e}", flush=True)
+        return False
+
     # (1a) v -> 2 v
     got = run_gpu(dict(x, v=x["v"] * 2), gpu_device, **kw)
     assert eq(got["y"], base["y"] * 2) and eq(got["lse"], base["lse"])
