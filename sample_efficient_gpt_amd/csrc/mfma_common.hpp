@@ -111,14 +111,17 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void* shared_obj) {
 // Completion is tracked by hand instead: wait_vmcnt<N>() followed by __syncthreads() publishes a stage.
 // (Hidden loads only make the compiler's own vmcnt waits conservative, never too weak: the counter
 // retires in order.)
+// On this architecture family an LDS-DMA instruction may not read M0 in the instruction slot right after a scalar
+// write to it (one wait state is required; the compiler inserts it for its own code but cannot see inside an
+// asm string), hence the s_nop: without it the load can, rarely, land at the previous destination.
 __device__ __forceinline__ void gload_lds16(const void* gsrc, uint32_t lds_dst_wave_uniform) {
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
                : "v"(gsrc), "s"(lds_dst_wave_uniform)
                : "memory", "m0");
 }
 __device__ __forceinline__ void gload_lds4(const void* gsrc, uint32_t lds_dst_wave_uniform) {
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off"
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
                :
                : "v"(gsrc), "s"(lds_dst_wave_uniform)
                : "memory", "m0");

@@ -186,7 +186,7 @@ def test_cfg3_full_size_exact_properties(gpu_device):
     got = run_gpu(xp, gpu_device, **kw)
     for n in ("y", "lse", "dq"):
         assert eq(got[n][:, :, :t], base[n][:, :, :t]), n
-        assert not eq(got[n][:, :, t:], base[n][:, :, t:]), n
+        assert not torch.equal(got[n][:, :, t:], base[n][:, :, t:]), n
     # (2b) new q, dO before token t
     xp = dict(x)
     for n in ("q", "d_o"):
@@ -195,7 +195,7 @@ def test_cfg3_full_size_exact_properties(gpu_device):
     got = run_gpu(xp, gpu_device, **kw)
     for n in ("dk", "dv"):
         assert eq(got[n][:, :, t:], base[n][:, :, t:]), n
-        assert not eq(got[n][:, :, :t], base[n][:, :, :t]), n
+        assert not torch.equal(got[n][:, :, :t], base[n][:, :, :t]), n
     # (3) reversed batch
     got = run_gpu({n: (v.flip(0) if n in ("q", "k", "v", "d_o") else v) for n, v in x.items()}, gpu_device, **kw)
     for n in ("y", "lse", "dq", "dk", "dv"):
