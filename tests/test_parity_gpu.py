@@ -850,3 +850,27 @@ def test_dropin_with_every_trailing_positional_equals_canonical_call(gpu_device)
     assert torch.equal(f["V"].grad, flat(t["v"].grad, Hkv)) and torch.equal(f["VF"].grad, flat(t["v_first"].grad, Hkv))
     for n in ("g_q", "g_k", "vr_coef", "gate_logits"):
         assert torch.equal(p[n].grad, t[n].grad), n
+
+
+def test_full_size_steps_repeat_bit_for_bit(gpu_device):
+    """100 forward + backward steps at the IMU-1 size on one set of buffers: every output of every step equals
+    the first step's bit for bit (no atomics, fixed reduction orders, and no stray LDS traffic)."""
+    from sample_efficient_gpt_amd.plan import AttnPlan
+
+    c = CONFIGS[3]
+    x = make_inputs(c, device=gpu_device)
+    plan = AttnPlan(x, eps=c.eps, sm_scale=c.sm_scale)
+    outs = [plan.y, plan.lse, plan.dq, plan.dk, plan.dv, plan.dg_q, plan.dg_k]
+    plan.forward()
+    plan.backward(kv_prepared=True)
+    torch.cuda.synchronize()
+    ref = [t.clone() for t in outs]
+    print("cfg3 repeatability", flush=True)
+    for it in range(100):
+        for t in outs[:5]:
+            t.zero_()
+        plan.forward()
+        plan.backward(kv_prepared=True)
+        torch.cuda.synchronize()
+        for name, a, b in zip(("y", "lse", "dq", "dk", "dv", "dg_q", "dg_k"), outs, ref):
+            assert torch.equal(a, b), f"step {it}: {name} differs from the first step"
