@@ -146,16 +146,22 @@ def test_cfg3_imu1_fwd_bwd_full_size(gpu_device):
     compare(run_gpu(xb, gpu_device, **kw), run_oracle(xb, **kw), c.dtype, names=["dg_q", "dg_k"], label="cfg3[b=0] ")
 
 
-def test_cfg3_full_size_exact_properties(gpu_device):
-    """Size-independent properties at the IMU-1 shape, all bit-exact: (1) scaling v or dO by a power of two
-    scales what is linear in them and leaves the rest alone; (2) causality: changing tokens >= t leaves the
-    outputs and dq of rows < t alone, changing queries / dO of rows < t leaves dk, dv of rows >= t alone;
-    (3) the batch entries are independent: reversing the batch reverses the results."""
-    c = CONFIGS[3]
+@pytest.mark.parametrize("cfg", [3, 4, 5])
+def test_full_size_exact_properties(gpu_device, cfg):
+    """Size-independent properties at the full benchmark shapes (IMU-1; S=8192 with gate and value residual;
+    head_dim 128), all bit-exact: (1) scaling v (and v_first) or dO by a power of two scales what is linear in
+    them and leaves the rest alone; (2) causality: changing tokens >= t leaves the outputs and dq of rows < t
+    alone, changing queries / dO of rows < t leaves dk, dv of rows >= t alone; (3) the batch entries are
+    independent: reversing the batch reverses the results."""
+    c = CONFIGS[cfg]
     x = make_inputs(c)
     kw = dict(eps=c.eps, sm_scale=c.sm_scale)
-    print("cfg3 exact properties", flush=True)
+    if c.extras:
+        kw["gate_scale"] = c.gate_scale
+    print(f"cfg{cfg} exact properties", flush=True)
     base = run_gpu(x, gpu_device, **kw)
+    per_token = ["q", "k", "v", "d_o"] + (["v_first"] if c.extras else [])
+    dvs = ["dv"] + (["dv_first"] if c.extras else [])
 
     def eq(a, b):
         a, b = a.float(), b.float()
@@ -166,23 +172,31 @@ def test_cfg3_full_size_exact_properties(gpu_device):
               f"max |diff| {float((a - b).abs().max()):.3e}", flush=True)
         return False
 
-    # (1a) v -> 2 v
-    got = run_gpu(dict(x, v=x["v"] * 2), gpu_device, **kw)
+    # (1a) v, v_first -> 2 v, 2 v_first
+    x2 = dict(x, v=x["v"] * 2)
+    if c.extras:
+        x2["v_first"] = x["v_first"] * 2
+    got = run_gpu(x2, gpu_device, **kw)
     assert eq(got["y"], base["y"] * 2) and eq(got["lse"], base["lse"])
-    assert eq(got["dq"], base["dq"] * 2) and eq(got["dk"], base["dk"] * 2) and eq(got["dv"], base["dv"])
+    assert eq(got["dq"], base["dq"] * 2) and eq(got["dk"], base["dk"] * 2)
+    for n in dvs:
+        assert eq(got[n], base[n]), n
     assert eq(got["dg_q"], base["dg_q"] * 2)
     # (1b) dO -> dO / 4
     got = run_gpu(dict(x, d_o=x["d_o"] * 0.25), gpu_device, **kw)
     assert eq(got["y"], base["y"])
-    for n in ("dq", "dk", "dv", "dg_q", "dg_k"):
+    for n in ["dq", "dk", "dg_q", "dg_k"] + dvs + (["dgate_logits", "dvr_coef"] if c.extras else []):
         assert eq(got[n], base[n] * 0.25), n
-    # (2a) new q, k, v, dO from token t on
-    t = 1111
+    # (2a) new q, k, v, dO (and gate logits) from token t on
+    t = c.S // 2 + 87
     g = torch.Generator().manual_seed(77)
     xp = dict(x)
-    for n in ("q", "k", "v", "d_o"):
+    for n in per_token:
         xp[n] = x[n].clone()
         xp[n][:, :, t:] = torch.randn(x[n][:, :, t:].shape, generator=g).to(x[n].dtype)
+    if c.extras:
+        xp["gate_logits"] = x["gate_logits"].clone()
+        xp["gate_logits"][:, t:] = torch.randn(x["gate_logits"][:, t:].shape, generator=g).to(x["gate_logits"].dtype)
     got = run_gpu(xp, gpu_device, **kw)
     for n in ("y", "lse", "dq"):
         assert eq(got[n][:, :, :t], base[n][:, :, :t]), n
@@ -193,12 +207,13 @@ def test_cfg3_full_size_exact_properties(gpu_device):
         xp[n] = x[n].clone()
         xp[n][:, :, :t] = torch.randn(x[n][:, :, :t].shape, generator=g).to(x[n].dtype)
     got = run_gpu(xp, gpu_device, **kw)
-    for n in ("dk", "dv"):
+    for n in ["dk"] + dvs:
         assert eq(got[n][:, :, t:], base[n][:, :, t:]), n
         assert not torch.equal(got[n][:, :, :t], base[n][:, :, :t]), n
     # (3) reversed batch
-    got = run_gpu({n: (v.flip(0) if n in ("q", "k", "v", "d_o") else v) for n, v in x.items()}, gpu_device, **kw)
-    for n in ("y", "lse", "dq", "dk", "dv"):
+    flipped = {n: (v.flip(0) if n in per_token + ["gate_logits"] else v) for n, v in x.items()}
+    got = run_gpu(flipped, gpu_device, **kw)
+    for n in ["y", "lse", "dq", "dk"] + dvs:
         assert eq(got[n].flip(0), base[n]), n
     assert torch.allclose(got["dg_q"], base["dg_q"], atol=2e-2, rtol=1e-2)
 
