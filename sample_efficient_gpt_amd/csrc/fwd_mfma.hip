@@ -41,18 +41,23 @@ constexpr float kLazyThresh = 16.f;   // general path: the subtracted reference 
 //   D(n)   mask (diagonal blocks only), exp2, bf16 pack, row sums
 //   A(n+1) request the row-major Khat fragments of block n+1 (possibly of the next tile, already landed)
 //   E(n)   O^T += V'^T P^T MFMAs
-template <int D>
+// Two shapes at head_dim 64.  WIDE: 64 query rows per wave (K fragments shared by two query blocks), four LDS
+// stages, two workgroups per CU: best when a workgroup streams many key tiles (S = 8192: 7 % faster than
+// NARROW).  NARROW: 32 rows per wave, three stages (48 KB), three workgroups per CU: twice as many, lighter
+// workgroups whose start-up / write-out latencies hide behind two neighbours instead of one (S = 2048: 1 %
+// faster, S = 1152: 10 %, S = 768: 13 %, S = 384: 27 %).  The launcher picks by the number of keys.
+template <int D, bool WIDE>
 struct FwdShape {
-  static constexpr int kNQB = D == 64 ? 2 : 1;     // 32-query blocks per wave
-  static constexpr int kStages = D == 64 ? 4 : 3;  // LDS: 64 KB (two workgroups per CU) / 96 KB
-  static constexpr int kOcc = D == 64 ? 2 : 1;
+  static constexpr int kNQB = (D == 64 && WIDE) ? 2 : 1;  // 32-query blocks per wave
+  static constexpr int kStages = D == 64 ? (WIDE ? 4 : 3) : 3;
+  static constexpr int kOcc = D == 64 ? (WIDE ? 2 : 3) : 1;
   static constexpr int kBQ = 4 * 32 * kNQB;
 };
 
-template <int D>
-__global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(KArgs a) {
+template <int D, bool WIDE>
+__global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16_kernel(KArgs a) {
   using Z = Swz<D>;
-  using F = FwdShape<D>;
+  using F = FwdShape<D, WIDE>;
   constexpr int NQB = F::kNQB, BQ = F::kBQ, NS = F::kStages;
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
@@ -300,19 +305,19 @@ __global__ __launch_bounds__(kThreadsM, FwdShape<D>::kOcc) void fwd_bf16_kernel(
   }
 }
 
-template <int D>
+template <int D, bool WIDE>
 int launch_fwd_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
-  const int n_qt = (p.Sq + FwdShape<D>::kBQ - 1) / FwdShape<D>::kBQ;
-  hipLaunchKernelGGL((fwd_bf16_kernel<D>), dim3((unsigned)(n_qt * p.H * p.B)), dim3(kThreadsM), 0, st, a);
+  const int n_qt = (p.Sq + FwdShape<D, WIDE>::kBQ - 1) / FwdShape<D, WIDE>::kBQ;
+  hipLaunchKernelGGL((fwd_bf16_kernel<D, WIDE>), dim3((unsigned)(n_qt * p.H * p.B)), dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 
 }  // namespace
 
 int launch_fwd_bf16(const KArgs& a, hipStream_t st) {
-  if (a.p.D == 64) return launch_fwd_t<64>(a, st);
-  if (a.p.D == 128) return launch_fwd_t<128>(a, st);
+  if (a.p.D == 64) return a.p.Sk > 2048 ? launch_fwd_t<64, true>(a, st) : launch_fwd_t<64, false>(a, st);
+  if (a.p.D == 128) return launch_fwd_t<128, true>(a, st);
   return (int)hipErrorInvalidValue;
 }
 
