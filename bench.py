@@ -35,7 +35,7 @@ MI355X_HBM_GBS = 8000.0
 # HBM bytes per launch (read + write) at cfg 3, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a plain
 # copy kernel of known size (FETCH_SIZE reads 0.5 of the true bytes on this part, WRITE_SIZE 1.0); profiler numbers,
 # not measured by this script
-PMC_TRAFFIC_BYTES_CFG3 = {"fwd": 117.1e6, "bwd_dq": 304.1e6, "bwd_dkdv": 195.0e6}
+PMC_TRAFFIC_BYTES_CFG3 = {"fwd": 118.8e6, "bwd_dq": 303.7e6, "bwd_dkdv": 198.4e6}
 
 
 def cpu_baseline(c, batches: int, budget_s: float = 12.0):
