@@ -1,7 +1,7 @@
 // bf16 forward: causal GQA flash attention on the normalised keys of the key/value pre-pass.
 //
-// Workgroup = 4 waves (two workgroups share a CU at head_dim 64 so that one's softmax overlaps the other's
-// MFMAs); wave w owns NQB blocks of 32 queries.  Scores are produced TRANSPOSED,
+// Workgroup = 4 waves (two or three workgroups share a CU at head_dim 64 so that one's softmax overlaps the
+// others' MFMAs); wave w owns NQB blocks of 32 queries (see FwdShape).  Scores are produced TRANSPOSED,
 //   S^T[key][query] = Khat[key][:] . Qhat[query][:]          (A = Khat tile from LDS, B = Qhat registers)
 // so every lane owns one query column: the softmax state (reference point, row sum) is a per-lane scalar,
 // row reductions are in-register plus one exchange with lane^32, and the bf16 probabilities are already
