@@ -97,6 +97,8 @@ def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scal
     lib = _lib.load()
     B, H, Sq, _ = q.shape
     lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    if q.numel() == 0:  # empty batch / no query rows: nothing to launch (the C ABI rejects zero sizes)
+        return lse, torch.empty(0, dtype=torch.uint8, device=q.device)
     p = _lib.new_params()
     _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope)
     kv_ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_KV, q.device)
@@ -118,6 +120,11 @@ def _backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_sca
     dg_q = torch.empty_like(g_q)
     dg_k = None if g_k is None else torch.empty_like(g_k)
     dcoef = None if vr_coef is None else torch.empty(2, dtype=torch.float32, device=dev)
+    if q.numel() == 0:  # no query rows: every gradient is zero
+        for t in (dq, dk, dv, dv_first, dgate, dg_q, dg_k, dcoef):
+            if t is not None:
+                t.zero_()
+        return dg_q, dg_k, dcoef
     p = _lib.new_params()
     _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope)
     p.d_o, p.dq, p.dk, p.dv = _lib.t4(dy), _lib.t4(dq), _lib.t4(dk), _lib.t4(dv)

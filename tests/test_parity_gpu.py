@@ -889,3 +889,22 @@ def test_full_size_steps_repeat_bit_for_bit(gpu_device):
         torch.cuda.synchronize()
         for name, a, b in zip(("y", "lse", "dq", "dk", "dv", "dg_q", "dg_k"), outs, ref):
             assert torch.equal(a, b), f"step {it}: {name} differs from the first step"
+
+
+def test_empty_batch_and_no_query_rows(gpu_device):
+    """B = 0 and Sq = 0: empty outputs, zero gradients, nothing launched (like torch's SDPA on empty inputs)."""
+    d = gpu_device
+    g = torch.ones(64, device=d, requires_grad=True)
+    for shape_q, shape_k in (((0, 4, 16, 64), (0, 2, 16, 64)), ((2, 4, 0, 64), (2, 2, 16, 64))):
+        q = torch.empty(shape_q, dtype=BF16, device=d, requires_grad=True)
+        k = torch.randn(shape_k, device=d).to(BF16).requires_grad_(True)
+        v = torch.randn(shape_k, device=d).to(BF16).requires_grad_(True)
+        y, lse = qknorm_attention(q, k, v, g, None, return_lse=True, causal=shape_q[2] != 0)
+        assert y.shape == shape_q and lse.shape == shape_q[:3]
+        y.sum().backward()
+        assert q.grad.shape == shape_q and torch.count_nonzero(k.grad) == 0 and torch.count_nonzero(v.grad) == 0
+        assert torch.count_nonzero(g.grad) == 0
+        g.grad = None
+    out = FlashAttnFunc.apply(torch.empty(0, 8, 64, dtype=BF16, device=d), torch.empty(0, 8, 64, dtype=BF16, device=d),
+                              torch.empty(0, 8, 64, dtype=BF16, device=d))
+    assert out.shape == (0, 8, 64)
