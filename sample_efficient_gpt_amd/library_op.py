@@ -64,7 +64,9 @@ def _(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scal
     lse = q.new_empty((B, H, Sq), dtype=torch.float32)
     # normalised keys (+ mixed values) of the bf16 path, rounded up to 256 bytes each; 256 bytes otherwise
     nbytes = 256
-    if q.dtype == torch.bfloat16:
+    if q.numel() == 0:
+        nbytes = 0
+    elif q.dtype == torch.bfloat16:
         piece = (k.shape[0] * k.shape[1] * k.shape[2] * D * 2 + 255) // 256 * 256
         nbytes = piece * (2 if v_first is not None else 1)
     return [y, lse, q.new_empty((nbytes,), dtype=torch.uint8)]
