@@ -24,9 +24,9 @@ def _case(device, dtype, B, H, Hkv, Sq, Sk, D, *, backward=True, seed=0, gen_kw=
     got = run_gpu(x, device, backward=backward, **kw)
     ref = run_oracle(x, backward=backward, **kw)
     scales = {}
-    if backward and dtype == BF16 and x["g_q"].numel() == 1:
+    if backward and x["g_q"].numel() == 1:
         scales.update(scalar_gain_scale(x, **kw))
-    if backward and dtype == BF16 and x.get("vr_coef") is not None:
+    if backward and x.get("vr_coef") is not None:
         scales.update(value_residual_scale(x, ref))
     return compare(got, ref, dtype, scales=scales or None, outliers=outliers)
 
