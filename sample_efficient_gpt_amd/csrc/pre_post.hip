@@ -1,9 +1,10 @@
-// HBM-bound helper kernels of the backward:
-//   bwd_pre     delta_i = rowsum(dY_i * Y_i); on the bf16 path also the normalised operands Qhat, Khat and
-//               V' that the two MFMA kernels stream (so their inner loops carry no norm arithmetic);
-//               with a gate also dgate = (1 - sigmoid(z)) * delta and
-//               dO_eff = gate_scale * sigmoid(z) * dY  (Y is the saved, already gated output, so
-//               rowsum(dO_eff * O) == rowsum(dY * Y) and no division by the gate is needed).
+// HBM-bound helper kernels:
+//   bwd_pre     (fp32 path) delta_i = rowsum(dY_i * Y_i); with a gate also dgate = (1 - sigmoid(z)) * delta
+//               and dO_eff = gate_scale * sigmoid(z) * dY  (Y is the saved, already gated output, so
+//               rowsum(dO_eff * O) == rowsum(dY * Y) and no division by the gate is needed).  On the bf16 path
+//               the dQ kernel's prologue does this.
+//   kv_prep     (bf16 path, forward and backward) the normalised keys Khat and mixed values V' that the MFMA
+//               kernels stream, so that their inner loops carry no norm arithmetic.
 //   bwd_reduce  second stage of the scale-gradient reduction: sums the per-workgroup partial
 //               vectors and applies dg_q = g_k * dg, dg_k = g_q * dg (the logits depend on the two
 //               scale vectors only through their product); also sums the (dc1, dc2) partials.
@@ -21,18 +22,6 @@ __global__ __launch_bounds__(256) void bwd_pre_kernel(KArgs a) {
   const int tid = threadIdx.x;
   const int part = tid % TPR;
   const int64_t nrows = (int64_t)p.B * p.H * p.Sq;
-  // the slice of the scale product this thread needs when it forms Qhat (bf16 path)
-  float gs[V];
-  if (a.qhat) {
-#pragma unroll
-    for (int e = 0; e < V; ++e) {
-      const int d = part * V + e;
-      float g = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
-      if (p.gk_numel == 1) g *= p.g_k[0];
-      else if (p.gk_numel > 1) g *= p.g_k[d];
-      gs[e] = g * p.sm_scale * kLog2e;
-    }
-  }
   for (int64_t row0 = (int64_t)blockIdx.x * RPB; row0 < nrows; row0 += (int64_t)gridDim.x * RPB) {
     const int64_t rid = row0 + tid / TPR;  // flat (b, h, s)
     const bool live = rid < nrows;
@@ -40,29 +29,15 @@ __global__ __launch_bounds__(256) void bwd_pre_kernel(KArgs a) {
     const int s = (int)(r % p.Sq);
     const int h = (int)((r / p.Sq) % p.H);
     const int b = (int)(r / ((int64_t)p.Sq * p.H));
-    float y[V], dy[V], q[V];
+    float y[V], dy[V];
     Elem<T>::load(row_ptr<T>(p.o, b, h, s) + part * V, y);
     Elem<T>::load(row_ptr<T>(p.d_o, b, h, s) + part * V, dy);
-    if (a.qhat) Elem<T>::load(row_ptr<T>(p.q, b, h, s) + part * V, q);
-    float acc = 0.f, ss = 0.f;
+    float acc = 0.f;
 #pragma unroll
     for (int e = 0; e < V; ++e) acc += y[e] * dy[e];
-    if (a.qhat) {
 #pragma unroll
-      for (int e = 0; e < V; ++e) ss += q[e] * q[e];
-    }
-#pragma unroll
-    for (int o = 1; o < TPR; o <<= 1) {
-      acc += __shfl_xor(acc, o, 64);
-      ss += __shfl_xor(ss, o, 64);
-    }
+    for (int o = 1; o < TPR; o <<= 1) acc += __shfl_xor(acc, o, 64);
     if (!live) continue;
-    if (a.qhat) {  // bf16 path: the normalised, scaled query row the two MFMA kernels consume
-      const float f = row_normaliser(p, ss, 1.0f / D);
-#pragma unroll
-      for (int e = 0; e < V; ++e) q[e] *= f * gs[e];
-      Elem<T>::store(reinterpret_cast<T*>(a.qhat) + r * D + part * V, q);
-    }
     if (part == 0) a.delta[r] = acc;
     if (p.gate.ptr) {
       const int64_t gi = (int64_t)b * p.gate.stride_b + (int64_t)s * p.gate.stride_s + (int64_t)h * p.gate.stride_h;
