@@ -44,10 +44,6 @@ __device__ __forceinline__ float norm_grad_coef(const segpt_attn_params& p, floa
   return (p.flags & SEGPT_FLAG_NO_NORM) ? 0.0f : n * n * n * inv_d;
 }
 
-struct __attribute__((aligned(16))) bf16x8_raw {
-  uint32_t w[4];
-};
-
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
 
 // round-to-nearest-even fp32 -> bf16 (inputs are finite in every use below)

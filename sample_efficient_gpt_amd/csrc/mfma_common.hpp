@@ -42,7 +42,6 @@ __device__ __forceinline__ float half_sum(float x) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float fast_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
 // acc + lo + hi of one packed bf16 pair (v_dot2c_f32_bf16 with a (1,1) operand): sums the ROUNDED values,
@@ -53,15 +52,6 @@ __device__ __forceinline__ float add_bf16_pair(uint32_t w, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, w), one, acc, false);
 }
 
-__device__ __forceinline__ float sumsq8(u32x4 v) {
-  float s = 0.f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float lo = bf16lo(v[i]), hi = bf16hi(v[i]);
-    s += lo * lo + hi * hi;
-  }
-  return s;
-}
 __device__ __forceinline__ u32x4 scale8(u32x4 v, float f) {
   u32x4 r;
 #pragma unroll
