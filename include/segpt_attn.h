@@ -175,6 +175,8 @@ const char* segpt_strerror(int code);
 
 /* Bytes of device scratch of kind `which` (SEGPT_WS_*) these params need (0 is possible). Validates
  * nothing but sizes; returns 0 for invalid params (the launch call will report the error).
+ * SEGPT_WS_KV follows p->flags: a decode-shaped forward with SEGPT_FLAG_DECODE needs only the split-key partial
+ * results (a small fraction of the cache), every other call the normalised keys (and mixed values).
  * Replaces the in-op allocations of triton_flash_attn_qknorm.py:286-287 / :320-323: the caller
  * allocates. */
 size_t segpt_attn_workspace_bytes(const segpt_attn_params* p, int which);

@@ -29,10 +29,22 @@ struct KvLayout {
   size_t khat, vmix, total;
 };
 
-// bf16 only: normalised keys and (with a value residual) mixed values, contiguous [B,Hkv,Sk,D]
+// A forward-only bf16 call with at most 32 query rows per kv head takes the split-key decode kernels when the
+// caller allows it with SEGPT_FLAG_DECODE; the kv workspace then holds partial results, not keys.
+bool decode_shape(const segpt_attn_params& p) {
+  return (p.flags & SEGPT_FLAG_DECODE) && p.dtype == SEGPT_DTYPE_BF16 && p.Hkv > 0 && (int64_t)(p.H / p.Hkv) * p.Sq <= 32;
+}
+
+// bf16 only: normalised keys and (with a value residual) mixed values, contiguous [B,Hkv,Sk,D]; for a decode-shaped
+// call the per-split partial results instead (a small fraction of the cache)
 KvLayout kv_layout(const segpt_attn_params& p) {
   KvLayout w{0, 0, 0};
   if (p.dtype != SEGPT_DTYPE_BF16) return w;
+  if (decode_shape(p)) {
+    int kend, splits, chunk;
+    w.total = align_up(decode_plan(p, &kend, &splits, &chunk));
+    return w;
+  }
   const size_t kvrows = (size_t)p.B * p.Hkv * p.Sk;
   size_t off = align_up(kvrows * p.D * 2);
   w.vmix = off;
@@ -72,6 +84,26 @@ int check_t4(const segpt_tensor4& t, const segpt_attn_params& p) {
   return SEGPT_OK;
 }
 
+// An OUTPUT view must not alias itself: with the extents (B, heads, rows) sorted by stride, every stride has to
+// step over the whole extent below it (a zero or too-small stride would make workgroups race on the same rows and
+// the call would still report success).  Extents of 1 are free.
+int check_t4_out(const segpt_tensor4& t, const segpt_attn_params& p, int heads, int rows) {
+  const int rc = check_t4(t, p);
+  if (rc) return rc;
+  int64_t st[3] = {t.stride_b, t.stride_h, t.stride_s};
+  int64_t ex[3] = {p.B, heads, rows};
+  for (int i = 0; i < 3; ++i)
+    for (int j = i + 1; j < 3; ++j)
+      if (st[j] < st[i]) { const int64_t a = st[i], b = ex[i]; st[i] = st[j]; ex[i] = ex[j]; st[j] = a; ex[j] = b; }
+  int64_t span = p.D;  // elements covered by everything below the current dimension
+  for (int i = 0; i < 3; ++i) {
+    if (ex[i] <= 1) continue;
+    if (st[i] < span) return SEGPT_E_STRIDE;
+    span = st[i] * ex[i];
+  }
+  return SEGPT_OK;
+}
+
 int check_common(const segpt_attn_params* p) {
   if (!p) return SEGPT_E_NULL;
   if (p->struct_bytes != sizeof(segpt_attn_params)) return SEGPT_E_STRUCT;
@@ -94,7 +126,6 @@ int check_common(const segpt_attn_params* p) {
   if ((rc = check_t4(p->q, *p))) return rc;
   if ((rc = check_t4(p->k, *p))) return rc;
   if ((rc = check_t4(p->v, *p))) return rc;
-  if ((rc = check_t4(p->o, *p))) return rc;
   if (p->v_first.ptr && (rc = check_t4(p->v_first, *p))) return rc;
   if (p->gate.ptr && (p->gate.stride_b < 0 || p->gate.stride_s < 0 || p->gate.stride_h < 0)) return SEGPT_E_STRIDE;
   if (p->rope_cos || p->rope_sin) {
@@ -122,15 +153,16 @@ void bind_kv(KArgs& a) {
 
 int check_bwd(const segpt_attn_params* p) {
   int rc;
+  if ((rc = check_t4(p->o, *p))) return rc;  // the saved output: an input here
   if ((rc = check_t4(p->d_o, *p))) return rc;
-  if ((rc = check_t4(p->dq, *p))) return rc;
-  if ((rc = check_t4(p->dk, *p))) return rc;
-  if ((rc = check_t4(p->dv, *p))) return rc;
+  if ((rc = check_t4_out(p->dq, *p, p->H, p->Sq))) return rc;
+  if ((rc = check_t4_out(p->dk, *p, p->Hkv, p->Sk))) return rc;
+  if ((rc = check_t4_out(p->dv, *p, p->Hkv, p->Sk))) return rc;
   if (!p->dg_q) return SEGPT_E_NULL;
   if (p->g_k && !p->dg_k) return SEGPT_E_EXTRAS;
   if (p->v_first.ptr) {
     if (!p->dv_first.ptr || !p->dvr_coef) return SEGPT_E_EXTRAS;
-    if ((rc = check_t4(p->dv_first, *p))) return rc;
+    if ((rc = check_t4_out(p->dv_first, *p, p->Hkv, p->Sk))) return rc;
   }
   if (p->gate.ptr) {
     if (!p->dgate.ptr) return SEGPT_E_EXTRAS;
@@ -179,18 +211,12 @@ size_t segpt_attn_workspace_bytes(const segpt_attn_params* p, int which) {
   return 0;
 }
 
-// A forward-only bf16 call with at most 32 query rows per kv head may take the split-key decode kernels
-// (the caller allows it with SEGPT_FLAG_DECODE; the kv workspace then holds partial results, not keys).
-static bool use_decode(const segpt_attn_params* p) {
-  if (!(p->flags & SEGPT_FLAG_DECODE) || p->dtype != SEGPT_DTYPE_BF16) return false;
-  if ((int64_t)(p->H / p->Hkv) * p->Sq > 32) return false;
-  int kend, splits, chunk;
-  return decode_plan(*p, &kend, &splits, &chunk) <= p->kv_workspace_bytes;
-}
+static bool use_decode(const segpt_attn_params* p) { return decode_shape(*p); }  // check_common sized the workspace for it
 
 static int fwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi, void* stream) {
   int rc = check_common(p);
   if (rc) return rc;
+  if ((rc = check_t4_out(p->o, *p, p->H, p->Sq))) return rc;
   KArgs a{};
   a.p = *p;
   bind_kv(a);
@@ -217,7 +243,11 @@ int segpt_attn_fwd_stage(const segpt_attn_params* p, int stage, void* stream) {
   return fwd_stage_impl(p, stage, stage, stream);
 }
 
-static int bwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi, void* stream) {
+static int bwd_stage_impl(const segpt_attn_params* p_in, int stage_lo, int stage_hi, void* stream) {
+  if (!p_in) return SEGPT_E_NULL;
+  segpt_attn_params p_copy = *p_in;
+  p_copy.flags &= ~SEGPT_FLAG_DECODE;  // a forward-only hint: the backward always works on normalised keys
+  const segpt_attn_params* p = &p_copy;
   int rc = check_common(p);
   if (rc) return rc;
   if ((rc = check_bwd(p))) return rc;

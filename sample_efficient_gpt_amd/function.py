@@ -20,6 +20,7 @@ own formula (triton_flash_attn_qknorm.py:67-91).
 from __future__ import annotations
 
 import math
+import threading
 
 import torch
 
@@ -101,9 +102,9 @@ def _forward(q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scal
         return lse, torch.empty(0, dtype=torch.uint8, device=q.device)
     p = _lib.new_params()
     _fill_common(p, q, k, v, y, lse, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope)
+    p.flags = flags | (_lib.SEGPT_FLAG_DECODE if inference else 0)  # before sizing: a decode-shaped call needs less
     kv_ws = _lib.alloc_workspace(lib, p, _lib.SEGPT_WS_KV, q.device)
     p.kv_workspace, p.kv_workspace_bytes = kv_ws.data_ptr(), kv_ws.numel()
-    p.flags = flags | (_lib.SEGPT_FLAG_DECODE if inference else 0)
     with torch.cuda.device(q.device):  # the launch goes to the tensors' device, whatever the current one is
         rc = lib.segpt_attn_fwd(p, torch.cuda.current_stream(q.device).cuda_stream)
     if rc != 0:
@@ -150,12 +151,39 @@ def _lastdim_contig(x):
     return x if x.stride(-1) == 1 else x.contiguous()
 
 
+def _no_backward_will_follow(*tensors):
+    """True when nothing can ask for a gradient of this call: grad mode is off (torch.no_grad / inference_mode,
+    as in the reference's generate loop, transformer.py:160) or no tensor input requires one.  Must be evaluated
+    by the CALLER of an autograd Function: inside ``forward`` grad mode is always off, and
+    ``ctx.needs_input_grad`` mirrors ``requires_grad`` even under no_grad (a Parameter gain keeps it True)."""
+    return (not torch.is_grad_enabled()) or not any(t is not None and t.requires_grad for t in tensors)
+
+
+class _GradModeAtApply:
+    """Mix-in for the positional drop-in Functions: records, in ``apply`` (the caller's context), whether a
+    backward can follow, for ``forward`` to read."""
+
+    _tls = threading.local()
+
+    @classmethod
+    def apply(cls, *args, **kwargs):
+        cls._tls.inference = _no_backward_will_follow(*(a for a in args if isinstance(a, torch.Tensor)))
+        try:
+            return super().apply(*args, **kwargs)
+        finally:
+            cls._tls.inference = False
+
+    @classmethod
+    def _inference(cls):
+        return bool(getattr(cls._tls, "inference", False))
+
+
 class _CoreFunc(torch.autograd.Function):
     """Canonical-layout op: q [B,H,Sq,D], k/v/v_first [B,Hkv,Sk,D], gate [B,Sq,H]."""
 
     @staticmethod
     def forward(ctx, q, k, v, g_q, g_k, v_first, vr_coef, gate, gate_scale, eps, sm_scale, causal, q_start, rope=None,
-                flags=0, out_bshd=False):
+                flags=0, out_bshd=False, inference=False):
         gq32, gk32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device)
         coef32 = None if vr_coef is None else vr_coef.detach().to(device=q.device, dtype=torch.float32).reshape(-1).contiguous()
         _check_inputs(q, k, v, gq32, gk32, v_first, coef32, gate)
@@ -171,7 +199,7 @@ class _CoreFunc(torch.autograd.Function):
             if y.stride(-1) != 1:
                 y = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, coef32, gate, gate_scale, eps, sm_scale, causal, q_start, y, rope,
-                              inference=not any(ctx.needs_input_grad), flags=flags)
+                              inference=inference, flags=flags)
         # the normalised keys (bf16 path) are kept for the backward: 1/rep of q's size
         ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate, y, lse, kv_ws)
         ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start, rope, flags)
@@ -197,7 +225,7 @@ class _CoreFunc(torch.autograd.Function):
             dg_k = dg_k.reshape(g_k.shape).to(g_k.dtype)
         if vr_coef is not None:
             dcoef = dcoef.reshape(vr_coef.shape).to(vr_coef.dtype)
-        return dq, dk, dv, dg_q, dg_k, dv_first, dcoef, dgate, None, None, None, None, None, None, None, None
+        return dq, dk, dv, dg_q, dg_k, dv_first, dcoef, dgate, None, None, None, None, None, None, None, None, None
 
 
 def qknorm_attention(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate_logits=None, gate_scale=2.0,
@@ -217,8 +245,9 @@ def qknorm_attention(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, gate
     ``y.permute(0, 2, 1, 3).reshape(B, Sq, H*D)`` is the ``b seq (h head_d)`` tensor of attention.py:243 without a copy.
     """
     rope = _rope_arg(rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, q_start, q.device, q.shape[-1])
+    inference = _no_backward_will_follow(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits)
     y, lse = _CoreFunc.apply(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
-                             rope, 0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM, out_bshd)
+                             rope, 0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM, out_bshd, inference)
     return (y, lse) if return_lse else y
 
 
@@ -228,7 +257,7 @@ def _canon(x, n_heads):
     return x.view(n_heads, n // n_heads, S, d).permute(1, 0, 2, 3)
 
 
-class QKNormFlashAttnFunc(torch.autograd.Function):
+class QKNormFlashAttnFunc(_GradModeAtApply, torch.autograd.Function):
     """Drop-in for ``TritonFlashAttnQKNormFunc`` (triton_flash_attn_qknorm.py:262-343).
 
     ``apply(Q, K, V, gain, is_causal=True, q_start=0, k_gain=None, v_first=None, vr_coef=None,
@@ -276,7 +305,7 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
         O = torch.empty_like(Q)
         rope = _rope_arg(rope_cos, rope_sin, None, 0, q_start, Q.device, Q.shape[-1])
         lse, kv_ws = _forward(q4, k4, v4, gq32, gk32, vf4, coef32, gate_logits, gate_scale, eps, sm_scale, is_causal,
-                              q_start, _canon(O, H), rope, inference=not any(ctx.needs_input_grad))
+                              q_start, _canon(O, H), rope, inference=QKNormFlashAttnFunc._inference())
         ctx.save_for_backward(lse, Q, K, V, gain, O, k_gain, v_first, vr_coef, gate_logits, kv_ws)
         ctx.cfg = (H, Hkv, gate_scale, eps, sm_scale, bool(is_causal), int(q_start), rope)
         return O
@@ -307,7 +336,24 @@ class QKNormFlashAttnFunc(torch.autograd.Function):
         return dQ, dK, dV, dgain, None, None, dk_gain, dVf, dcoef, dgate, None, None, None, None, None, None
 
 
-class FlashAttnFunc(torch.autograd.Function):
+class TritonFlashAttnQKNormFunc(QKNormFlashAttnFunc):
+    """The reference's class name WITH the reference kernel's own formula as the default
+    (triton_flash_attn_qknorm.py:67-91: L2 normaliser ``rsqrt(sum x^2 + 1e-8)``, logits ``gain * cos``), i.e. the
+    family at ``eps = 1e-8 / d, sm_scale = 1 / d``.  ``QKNormFlashAttnFunc`` keeps the live module's defaults
+    (RMS normaliser, eps 1e-6, 1/sqrt(d); attention.py:51-80).  Same positional signature; explicit ``eps`` /
+    ``sm_scale`` override the defaults."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, gain, is_causal=True, q_start=0, k_gain=None, v_first=None, vr_coef=None,
+                gate_logits=None, gate_scale=2.0, n_kv_heads=None, eps=None, sm_scale=None, rope_cos=None,
+                rope_sin=None):
+        d = Q.shape[-1]
+        return QKNormFlashAttnFunc.forward(ctx, Q, K, V, gain, is_causal, q_start, k_gain, v_first, vr_coef, gate_logits,
+                                           gate_scale, n_kv_heads, 1e-8 / d if eps is None else eps,
+                                           1.0 / d if sm_scale is None else sm_scale, rope_cos, rope_sin)
+
+
+class FlashAttnFunc(_GradModeAtApply, torch.autograd.Function):
     """Drop-in for the reference's attention WITHOUT QK-norm, ``TritonFlashAttnFunc``
     (triton_flash_attn.py:208-297; called at attention.py:240): ``apply(Q, K, V, q_start=0, is_causal=True,
     n_kv_heads=None)`` -- note the argument order, which differs from the QK-norm op's.  ``Q [(h b), Nq, d]``,
@@ -337,7 +383,7 @@ class FlashAttnFunc(torch.autograd.Function):
         sm_scale = 1.0 / math.sqrt(Q.shape[-1])
         O = torch.empty_like(Q)
         lse, kv_ws = _forward(q4, k4, v4, one, None, None, None, None, 1.0, 0.0, sm_scale, is_causal, q_start, _canon(O, H),
-                              None, inference=not any(ctx.needs_input_grad), flags=_lib.SEGPT_FLAG_NO_NORM)
+                              None, inference=FlashAttnFunc._inference(), flags=_lib.SEGPT_FLAG_NO_NORM)
         ctx.save_for_backward(lse, Q, K, V, O, one, kv_ws)
         ctx.cfg = (H, Hkv, sm_scale, bool(is_causal), int(q_start))
         return O

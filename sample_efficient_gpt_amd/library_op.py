@@ -5,11 +5,13 @@ non-reentrant activation checkpointing (transformer/transformer.py:123-132) as O
 
     y = torch.ops.segpt.qknorm_attention(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits,
                                          gate_scale, eps, sm_scale, causal, q_start,
-                                         rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm, out_bshd)[0]
+                                         rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm, out_bshd,
+                                         inference)[0]
 
 or the keyword wrapper ``qknorm_attention_op(...)`` below.  Canonical layout: q ``[B,H,Sq,D]``, k / v /
 v_first ``[B,Hkv,Sk,D]`` (any strides, last dim contiguous), gate_logits ``[B,Sq,H]``; the optional tensors
-are ``None`` when unused (rope_q_pos0 = -1 means "q_start").  Returns ``(y, lse, kv_ws)``: the output, the fp32 log-sum-exp ``[B,H,Sq]`` and the
+are ``None`` when unused (rope_q_pos0 = -1 means "q_start"); ``inference=True`` promises that no backward
+follows (decode-shaped calls may then take the split-key kernels, whose key/value workspace holds no keys).  Returns ``(y, lse, kv_ws)``: the output, the fp32 log-sum-exp ``[B,H,Sq]`` and the
 key/value workspace the backward reuses.  Same kernels and C ABI as ``function.py``; no fallback.
 """
 
@@ -22,7 +24,8 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .function import _backward, _check_inputs, _forward, _lastdim_contig, _rope_arg, _scale_arg
+from .function import (_backward, _check_inputs, _forward, _lastdim_contig, _no_backward_will_follow, _rope_arg,
+                       _scale_arg)
 
 __all__ = ["qknorm_attention_op"]
 
@@ -44,7 +47,7 @@ def _coef32(vr_coef, device):
 def _fwd_op(q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optional[Tensor], v_first: Optional[Tensor],
             vr_coef: Optional[Tensor], gate_logits: Optional[Tensor], gate_scale: float, eps: float, sm_scale: float,
             causal: bool, q_start: int, rope_cos: Optional[Tensor], rope_sin: Optional[Tensor],
-            rope_q_pos0: int, rope_k_pos0: int, qk_norm: bool, out_bshd: bool) -> List[Tensor]:
+            rope_q_pos0: int, rope_k_pos0: int, qk_norm: bool, out_bshd: bool, inference: bool) -> List[Tensor]:
     rope = _rope_arg(rope_cos, rope_sin, None if rope_q_pos0 < 0 else rope_q_pos0, rope_k_pos0, q_start, q.device, q.shape[-1])
     gq32, gk32, c32 = _scale_arg(g_q, q.device), _scale_arg(g_k, q.device), _coef32(vr_coef, q.device)
     _check_inputs(q, k, v, gq32, gk32, v_first, c32, gate_logits)
@@ -52,19 +55,21 @@ def _fwd_op(q: Tensor, k: Tensor, v: Tensor, g_q: Tensor, g_k: Optional[Tensor],
     v_first = None if v_first is None else _lastdim_contig(v_first)
     y = _empty_out(q, out_bshd)
     lse, kv_ws = _forward(q, k, v, gq32, gk32, v_first, c32, gate_logits, gate_scale, eps, sm_scale, causal, q_start, y, rope,
-                          flags=0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM)
+                          inference=inference, flags=0 if qk_norm else _lib.SEGPT_FLAG_NO_NORM)
+    if inference:  # no backward will read it (and after the decode kernels it holds no keys)
+        kv_ws = q.new_empty((0,), dtype=torch.uint8)
     return [y, lse, kv_ws]
 
 
 @_fwd_op.register_fake
 def _(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
-      rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm, out_bshd):
+      rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm, out_bshd, inference):
     B, H, Sq, D = q.shape
     y = _empty_out(q, out_bshd)
     lse = q.new_empty((B, H, Sq), dtype=torch.float32)
     # normalised keys (+ mixed values) of the bf16 path, rounded up to 256 bytes each; 256 bytes otherwise
     nbytes = 256
-    if q.numel() == 0:
+    if q.numel() == 0 or inference:
         nbytes = 0
     elif q.dtype == torch.bfloat16:
         piece = (k.shape[0] * k.shape[1] * k.shape[2] * D * 2 + 255) // 256 * 256
@@ -114,7 +119,7 @@ def _(dy, q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, gate_
 
 def _setup_context(ctx, inputs, output):
     (q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, gate_scale, eps, sm_scale, causal, q_start,
-     rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm, out_bshd) = inputs
+     rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm, out_bshd, _inference) = inputs
     y, lse, kv_ws = output
     ctx.save_for_backward(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, y, lse, kv_ws, rope_cos, rope_sin)
     ctx.cfg = (gate_scale, eps, sm_scale, causal, q_start, rope_q_pos0, rope_k_pos0, qk_norm)
@@ -129,7 +134,7 @@ def _autograd_backward(ctx, grads):
         rope_cos, rope_sin, rope_q_pos0, rope_k_pos0, qk_norm)
     return (dq, dk, dv, dg_q, None if g_k is None else dg_k, None if v_first is None else dvf,
             None if vr_coef is None else dcoef, None if gate_logits is None else dgate, None, None, None, None, None,
-            None, None, None, None, None, None)
+            None, None, None, None, None, None, None)
 
 
 _fwd_op.register_autograd(_autograd_backward, setup_context=_setup_context)
@@ -141,8 +146,11 @@ def qknorm_attention_op(q, k, v, g_q, g_k=None, *, v_first=None, vr_coef=None, g
     """Keyword front end of ``torch.ops.segpt.qknorm_attention`` (same arguments as ``qknorm_attention``)."""
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
+    # decided here, in the caller's grad mode: a forward-only call (the reference's generate loop runs under
+    # inference_mode, transformer.py:160) with few query rows takes the split-key decode kernels
+    inference = _no_backward_will_follow(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits)
     y, lse, _ = torch.ops.segpt.qknorm_attention(q, k, v, g_q, g_k, v_first, vr_coef, gate_logits, float(gate_scale),
                                                  float(eps), float(sm_scale), bool(causal), int(q_start),
                                                  rope_cos, rope_sin, -1 if rope_q_pos0 is None else int(rope_q_pos0),
-                                                 int(rope_k_pos0), bool(qk_norm), bool(out_bshd))
+                                                 int(rope_k_pos0), bool(qk_norm), bool(out_bshd), bool(inference))
     return (y, lse) if return_lse else y

@@ -45,6 +45,8 @@ class KVCache:
         self.length = 0
         self._cap = int(capacity)
         self._kbuf = self._vbuf = None
+        self._mbuf = None  # mixed values c1 v + c2 v_first of the layer that hands them on as v1 (filled on demand)
+        self._mlen = 0
 
     def append(self, k, v):
         B, Hkv, S, D = k.shape
@@ -62,6 +64,22 @@ class KVCache:
         self.length = need
         self.keys, self.values = self._kbuf[:, :, :need], self._vbuf[:, :, :need]
         return self.keys, self.values
+
+    def append_mixed(self, vm_new):
+        """Rows [length - S, length) of the mixed value tensor (the ``V`` a value-residual layer returns for later
+        layers, attention.py:228,267), kept beside the raw values so that a generation step mixes only its new
+        rows instead of the whole cache.  Call after ``append`` of the same step; returns the ``[B, Hkv, length, D]``
+        view."""
+        S = vm_new.shape[2]
+        assert self._mlen + S == self.length, "append_mixed follows append, once per step"
+        if self._mbuf is None or self._mbuf.shape[2] < self._vbuf.shape[2]:
+            mb = torch.empty_like(self._vbuf)
+            if self._mbuf is not None:
+                mb[:, :, : self._mlen].copy_(self._mbuf[:, :, : self._mlen])
+            self._mbuf = mb
+        self._mbuf[:, :, self._mlen : self.length].copy_(vm_new)
+        self._mlen = self.length
+        return self._mbuf[:, :, : self.length]
 
 
 class _Linear(nn.Module):
@@ -90,7 +108,9 @@ class MultiHeadSelfAttention(nn.Module):
     folded into the V loads, the per-head gate into the output write, and the output lands in ``b seq (h d)``
     layout for the output projection.  ``kv_cache`` is this package's ``KVCache`` (raw, un-expanded keys).
 
-    Differences a caller can see: the returned ``V`` (the tensor later layers take as ``v1``, attention.py:267) is
+    Differences a caller can see: a layer that is handed ``v1`` returns ``None`` as its second output unless
+    ``always_return_values`` is set (the reference's model only ever uses the first layer's, transformer.py:135-136);
+    the returned ``V`` (the tensor later layers take as ``v1``, attention.py:267) is
     the mixed value tensor as an un-expanded ``[b, hkv, Sk, d]`` view (the reference returns the flattened,
     ``repeat_interleave``-expanded ``[(h b), Sk, d]`` one, whose rows are equal within a GQA group); ``v1`` is
     accepted in that layout, in the reference's, and as ``[(hkv b), Sk, d]``.  As in the reference, ``token_positions`` is not used (positions follow from the cache length,
@@ -131,6 +151,10 @@ class MultiHeadSelfAttention(nn.Module):
             self.register_buffer("alpha1", torch.tensor([1.0], device=device), persistent=False)
             self.register_buffer("alpha2", torch.tensor([0.0], device=device), persistent=False)
             self.register_buffer("scale", torch.tensor([1.0], device=device), persistent=False)
+        # attention.py:267 returns the mixed V from every layer, but only the first layer's is ever used
+        # (transformer.py:135-136: `if v1 is None: v1 = v`).  False: layers that are GIVEN v1 return None instead
+        # of spending an elementwise pass (over the whole cache at generation time) on a tensor nobody reads.
+        self.always_return_values = False
         self.gating = gating
         if gating:
             gate_in, gate_out = {"elementwise": (d_model, d_model), "per-head": (d_model, n_heads),
@@ -158,7 +182,7 @@ class MultiHeadSelfAttention(nn.Module):
             k, v = kv_cache.append(k, v)
         Sk = k.shape[2]
         v_first = vr_coef = None
-        v_mixed = v
+        v_mixed = v if v1 is None or self.always_return_values else None
         if self.value_residual:  # attention.py:222-228; with the buffers (1, 0, 1) the line is the identity in fp32
             if v1 is None:
                 v_first = v
@@ -170,8 +194,15 @@ class MultiHeadSelfAttention(nn.Module):
                 v_first = _canon(v1.reshape(H * b, Sk, d), H)[:, :: H // Hkv]
             n = torch.rsqrt(self.alpha1**2 + self.alpha2**2 + 1e-8)
             vr_coef = torch.cat([self.scale * self.alpha1 * n, self.scale * self.alpha2 * n]).float()
-            c = vr_coef.to(v.dtype)
-            v_mixed = c[0] * v + c[1] * v_first  # only the returned tensor: the kernel mixes on its own
+            # The returned tensor only (the kernel mixes on its own, in fp32): built when a later layer can take it
+            # as v1, with fp32 coefficients like the reference's promotion (attention.py:228), and, during cached
+            # generation, for the new rows only.
+            if v_mixed is not None:
+                mix = lambda a, f: (vr_coef[0] * a.float() + vr_coef[1] * f.float()).to(v.dtype)
+                if kv_cache is not None and v1 is None and not torch.is_grad_enabled():
+                    v_mixed = kv_cache.append_mixed(mix(v[:, :, q_start:], v_first[:, :, q_start:]))
+                else:
+                    v_mixed = mix(v, v_first)
         gate_logits = None
         if self.gating == "per-head":
             gate_logits = self.attn_gate(x)

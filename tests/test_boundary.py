@@ -91,6 +91,17 @@ def test_argument_errors_are_reported_before_any_launch(lib):
     assert lib.segpt_attn_fwd(p, None) == -6
     p = _valid_params(); p.k.stride_h = 7
     assert lib.segpt_attn_fwd(p, None) == -6
+    # an OUTPUT view must not alias itself (a broadcast or overlapping view would make workgroups race)
+    p = _valid_params(); p.o.stride_h = 0
+    assert lib.segpt_attn_fwd(p, None) == -6
+    p = _valid_params(); p.o.stride_b = 128 * 64  # batches overlap the heads
+    assert lib.segpt_attn_fwd(p, None) == -6
+    p = _valid_params(); p.workspace, p.workspace_bytes = 0x20000, 1 << 30
+    p.dq.stride_b = 0
+    assert lib.segpt_attn_bwd(p, None) == -6
+    p = _valid_params(); p.workspace, p.workspace_bytes = 0x20000, 1 << 30
+    p.dk = _lib.Tensor4(0x10000, 2 * 128 * 64, 64, 64)  # heads interleaved at the row pitch: rows collide
+    assert lib.segpt_attn_bwd(p, None) == -6
     p = _valid_params(); p.q_start = -1
     assert lib.segpt_attn_fwd(p, None) == -9
     p = _valid_params(); p.v.ptr = 0x10004
@@ -173,8 +184,14 @@ def test_function_signature_is_the_reference_one():
     assert sig.parameters["is_causal"].default is True and sig.parameters["q_start"].default == 0
     for extra in names[7:]:
         assert sig.parameters[extra].default is not inspect.Parameter.empty  # extras are optional
-    assert TritonFlashAttnQKNormFunc is QKNormFlashAttnFunc
     assert issubclass(QKNormFlashAttnFunc, torch.autograd.Function)
+    # the reference's own name: same positional signature, but its defaults are the reference KERNEL's formula
+    # (eps = 1e-8 / d on the mean, logits gain * cos; triton_flash_attn_qknorm.py:67-91), resolved at call time
+    assert issubclass(TritonFlashAttnQKNormFunc, QKNormFlashAttnFunc)
+    ref_sig = inspect.signature(TritonFlashAttnQKNormFunc.forward)
+    assert list(ref_sig.parameters) == names
+    assert ref_sig.parameters["eps"].default is None and ref_sig.parameters["sm_scale"].default is None
+    assert sig.parameters["eps"].default == 1e-6 and sig.parameters["sm_scale"].default is None
 
 
 def test_function_asserts_like_the_reference_on_host_tensors():
@@ -226,7 +243,7 @@ def test_library_op_is_registered_with_a_shape_only_implementation():
     with FakeTensorMode():  # what torch.compile sees: device tensors without storage
         dev = lambda *s, dt=torch.bfloat16: torch.empty(*s, dtype=dt, device="cuda")
         out = torch.ops.segpt.qknorm_attention(dev(1, 4, 50, 128), dev(1, 2, 70, 128), dev(1, 2, 70, 128), dev(1, dt=torch.float32),
-                                               None, dev(1, 2, 70, 128), dev(2, dt=torch.float32), dev(1, 50, 4), 2.0, 1e-6, 0.1, True, 20, None, None, -1, 0, True, False)
+                                               None, dev(1, 2, 70, 128), dev(2, dt=torch.float32), dev(1, 50, 4), 2.0, 1e-6, 0.1, True, 20, None, None, -1, 0, True, False, False)
         assert out[0].shape == (1, 4, 50, 128) and out[1].shape == (1, 4, 50)
         assert out[2].numel() == 2 * (2 * 70 * 128 * 2 + 255) // 256 * 256 or out[2].numel() >= 2 * 2 * 70 * 128 * 2
 

@@ -28,7 +28,28 @@ def _case(device, dtype, B, H, Hkv, Sq, Sk, D, *, backward=True, seed=0, gen_kw=
         scales.update(scalar_gain_scale(x, **kw))
     if backward and x.get("vr_coef") is not None:
         scales.update(value_residual_scale(x, ref))
-    return compare(got, ref, dtype, scales=scales or None, outliers=outliers)
+    if dtype == BF16 and backward:
+        _fp32_proof(device, x, ref, kw)
+    try:
+        return compare(got, ref, dtype, scales=scales or None)
+    except AssertionError:
+        if outliers is None:
+            raise
+        # Allowance for isolated elements: granted only to a case whose mathematics the fp32 kernels have just
+        # reproduced at 1e-5 on the same inputs (_fp32_proof above), so that what is left is bf16 rounding noise.
+        print("strict bound exceeded; fp32 kernels agree with the oracle at 1e-5 on this case: applying the outlier allowance", flush=True)
+        return compare(got, ref, dtype, scales=scales or None, outliers=outliers)
+
+
+def _fp32_proof(device, x, ref, kw, backward=True):
+    """The bf16 comparisons use magnitude yardsticks for gradients that are sums over every row (and, in the sweep,
+    an allowance for isolated elements).  They are only meaningful if the slack they grant is bf16 rounding noise and
+    not a wrong formula, so every such case also runs the fp32 kernels on the SAME inputs (the bf16 values, widened)
+    and asserts 1e-5 against the same oracle result, every output and gradient, element-wise for the tensors and
+    relative to the largest entry for the summed parameter gradients."""
+    x32 = {n: (t.float() if torch.is_tensor(t) and t.dtype == BF16 else t) for n, t in x.items()}
+    got32 = run_gpu(x32, device, backward=backward, **kw)
+    compare(got32, ref, F32, label="fp32 kernels on the same inputs: ")
 
 
 # ------------------------------------------------------------------ fp32 path (1e-5)
@@ -91,22 +112,34 @@ def test_bf16_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
     _case(gpu_device, BF16, B, H, Hkv, Sq, Sk, D, gen_kw=gen_kw, **kw)
 
 
+def _slice_inputs(c, x, b, g):
+    rep = c.H // c.Hkv
+    hs = slice(g * rep, (g + 1) * rep)
+    xs = {"q": x["q"][b:b + 1, hs], "k": x["k"][b:b + 1, g:g + 1], "v": x["v"][b:b + 1, g:g + 1],
+          "d_o": x["d_o"][b:b + 1, hs], "g_q": x["g_q"], "g_k": x["g_k"]}
+    if c.extras:
+        xs.update(gate_logits=x["gate_logits"][b:b + 1, :, hs], v_first=x["v_first"][b:b + 1, g:g + 1], vr_coef=x["vr_coef"])
+    return xs, hs
+
+
+REDUCED_GRADS = ("dg_q", "dg_k", "dvr_coef")
+
+
 def _slice_check(device, c, pairs, odtype=torch.float64):
-    """Full-size run on the GPU; oracle on single (batch, kv-group) slices (they are independent)."""
+    """Full-size run on the GPU; oracle on single (batch, kv-group) slices (they are independent units).
+    Tensors: the full run's slice against the oracle's.  Parameter gradients that sum over every row
+    (dg_q, dg_k, dvr_coef): (i) a GPU run on the slice alone against the oracle's slice result, (ii) the full run's
+    value against the sum of GPU runs over ALL (batch, kv-group) slices (the reduction is additive over them), so
+    that a wrong partial, a dropped workgroup or a wrong second-stage reduce at full size fails."""
     x = make_inputs(c)
     kw = dict(eps=c.eps, sm_scale=c.sm_scale)
     if c.extras:
         kw["gate_scale"] = c.gate_scale
     print(f"full-size {c.name}", flush=True)
     got = run_gpu(x, device, backward=c.backward, **kw)
-    rep = c.H // c.Hkv
     worst = {}
     for b, g in pairs:
-        hs = slice(g * rep, (g + 1) * rep)
-        xs = {"q": x["q"][b:b + 1, hs], "k": x["k"][b:b + 1, g:g + 1], "v": x["v"][b:b + 1, g:g + 1],
-              "d_o": x["d_o"][b:b + 1, hs], "g_q": x["g_q"], "g_k": x["g_k"]}
-        if c.extras:
-            xs.update(gate_logits=x["gate_logits"][b:b + 1, :, hs], v_first=x["v_first"][b:b + 1, g:g + 1], vr_coef=x["vr_coef"])
+        xs, hs = _slice_inputs(c, x, b, g)
         ref = run_oracle(xs, backward=c.backward, odtype=odtype, **kw)
         gs = {"y": got["y"][b:b + 1, hs], "lse": got["lse"][b:b + 1, hs]}
         names = ["y", "lse"]
@@ -117,9 +150,30 @@ def _slice_check(device, c, pairs, odtype=torch.float64):
                 gs.update(dv_first=got["dv_first"][b:b + 1, g:g + 1], dgate_logits=got["dgate_logits"][b:b + 1, :, hs])
                 names += ["dv_first", "dgate_logits"]
         errs = compare(gs, ref, c.dtype, names=names, label=f"{c.name}[b={b},g={g}] ")
+        if c.backward:  # (i) the summed parameter gradients of this slice, GPU alone on the slice vs the oracle
+            alone = run_gpu(xs, device, **kw)
+            red = [n for n in REDUCED_GRADS if n in ref]
+            scales = value_residual_scale(xs, ref) if c.extras else None
+            errs.update(compare(alone, ref, c.dtype, names=red, label=f"{c.name}[b={b},g={g}] slice alone ", scales=scales))
         for n, e in errs.items():
             worst[n] = max(worst.get(n, 0.0), e)
     print(c.name, "worst max-abs errors over slices:", {k: f"{v:.2e}" for k, v in worst.items()}, flush=True)
+    if c.backward:  # (ii) additivity over every (batch, kv-group) slice
+        red = [n for n in REDUCED_GRADS if n in got]
+        acc = {n: torch.zeros_like(got[n], dtype=torch.float64) for n in red}
+        mag = {n: torch.zeros_like(got[n], dtype=torch.float64) for n in red}
+        for b in range(c.B):
+            for g in range(c.Hkv):
+                part = run_gpu(_slice_inputs(c, x, b, g)[0], device, **kw)
+                for n in red:
+                    acc[n] += part[n].double()
+                    mag[n] += part[n].double().abs()
+        for n in red:
+            # both sides are fp32 sums of the same per-workgroup partials in different orders: only fp32 summation
+            # noise separates them (1e-4 of the summed magnitudes is ~100x that noise and ~100x below the bf16 budget)
+            err = (got[n].double() - acc[n]).abs()
+            assert bool((err <= 1e-5 + 1e-4 * mag[n]).all()), f"{c.name} {n}: full run {got[n]} vs sum of slices {acc[n]}"
+            print(f"{c.name} {n}: full run vs sum over {c.B * c.Hkv} slices, max abs diff {float(err.max()):.3e}", flush=True)
     return x, got, kw
 
 
@@ -128,22 +182,7 @@ def test_cfg2_imu1_forward_full_size(gpu_device):
 
 
 def test_cfg3_imu1_fwd_bwd_full_size(gpu_device):
-    c = CONFIGS[3]
-    x, got, kw = _slice_check(gpu_device, c, [(0, 0), (7, 5)])
-    # the scale-vector gradients sum over every (b, h, row): check them as a sum of per-batch GPU runs
-    # (additivity), each of which the small cases above compare with the oracle
-    acc_q = torch.zeros(c.D, dtype=torch.float64)
-    acc_k = torch.zeros(c.D, dtype=torch.float64)
-    for b in range(c.B):
-        xb = {n: (t[b:b + 1] if n in ("q", "k", "v", "d_o") else t) for n, t in x.items()}
-        gb = run_gpu(xb, gpu_device, **kw)
-        acc_q += gb["dg_q"].double()
-        acc_k += gb["dg_k"].double()
-    assert torch.allclose(got["dg_q"].double(), acc_q, atol=2e-2, rtol=1e-2)
-    assert torch.allclose(got["dg_k"].double(), acc_k, atol=2e-2, rtol=1e-2)
-    # and one batch of it directly against the oracle
-    xb = {n: (t[:1] if n in ("q", "k", "v", "d_o") else t) for n, t in x.items()}
-    compare(run_gpu(xb, gpu_device, **kw), run_oracle(xb, **kw), c.dtype, names=["dg_q", "dg_k"], label="cfg3[b=0] ")
+    _slice_check(gpu_device, CONFIGS[3], [(0, 0), (7, 5)])
 
 
 @pytest.mark.parametrize("cfg", [3, 4, 5])
@@ -256,6 +295,7 @@ def test_running_maximum_path(gpu_device):
     ref = run_oracle(x, backward=False)
     # the bf16 rounding of Qhat and Khat perturbs a logit in proportion to the gain product (5.8x the ordinary
     # case here), and P = exp(logit) inherits it: the absolute part of the tolerance is scaled accordingly
+    _fp32_proof(gpu_device, x, ref, {}, backward=False)  # the fp32 kernels meet 1e-5 on these inputs: the slack below is rounding
     err = (got["y"].double() - ref["y"]).abs()
     assert bool((err <= 5.8 * 2e-2 + 1e-2 * ref["y"].abs()).all()), float(err.max())
     assert torch.allclose(got["lse"].double(), ref["lse"], atol=5.8 * 2e-2, rtol=1e-2)
@@ -323,7 +363,7 @@ def test_library_op_compiled_and_checkpointed_matches_eager(gpu_device):
         for a, b in zip(ref, other):
             assert torch.equal(a, b)
     torch.library.opcheck(torch.ops.segpt.qknorm_attention,
-                          tuple(x[n].to(gpu_device) for n in names) + (2.0, 1e-6, 0.125, True, 0, None, None, -1, 0, True, False),
+                          tuple(x[n].to(gpu_device) for n in names) + (2.0, 1e-6, 0.125, True, 0, None, None, -1, 0, True, False, False),
                           test_utils=("test_schema", "test_faketensor"))
     # every optional operand absent: the backward op then returns several empty placeholders, which must be
     # distinct tensors (returns of a custom op may not alias one another)
@@ -571,6 +611,81 @@ def test_fused_triton_formula_is_reachable_variant_b(gpu_device):
     compare({"y": out.cpu()}, {"y": O_ref}, F32)
 
 
+def test_reference_named_function_defaults_to_the_reference_kernel_formula(gpu_device):
+    """`TritonFlashAttnQKNormFunc.apply(Q, K, V, gain)` with NO further arguments computes what the reference class of
+    that name computes (triton_flash_attn_qknorm.py:67-91: L2 normaliser with 1e-8 on the sum, logits gain*cos), not
+    the live module's 1/sqrt(d)-scaled RMS form; forward and the gradients of Q, K, V and the gain."""
+    from sample_efficient_gpt_amd import TritonFlashAttnQKNormFunc
+
+    S, D = 96, 64
+    x = gen(2, 1, 1, S, S, D, F32, scalar_gain=True, no_gk=True, seed=19)
+    Q, K, V, dO = (x[n][:, 0].contiguous() for n in ("q", "k", "v", "d_o"))
+    ref_in = [t.double().requires_grad_(True) for t in (Q, K, V, x["g_q"])]
+    O_ref, _ = orc.fused_kernel_variant_b(*ref_in)
+    O_ref.backward(dO.double())
+    d = gpu_device
+    dev_in = [t.to(d).requires_grad_(True) for t in (Q, K, V, x["g_q"])]
+    out = TritonFlashAttnQKNormFunc.apply(*dev_in)
+    out.backward(dO.to(d))
+    compare({"y": out.detach().cpu(), "dq": dev_in[0].grad.cpu(), "dk": dev_in[1].grad.cpu(), "dv": dev_in[2].grad.cpu(),
+             "dg_q": dev_in[3].grad.cpu()},
+            {"y": O_ref.detach(), "dq": ref_in[0].grad, "dk": ref_in[1].grad, "dv": ref_in[2].grad, "dg_q": ref_in[3].grad}, F32)
+    # and it differs from the live-module defaults of QKNormFlashAttnFunc (logits sqrt(d) times larger there)
+    live = QKNormFlashAttnFunc.apply(*(t.detach() for t in dev_in))
+    assert float((live.cpu().double() - O_ref.detach()).abs().max()) > 1e-2
+
+
+@pytest.mark.parametrize("dtype,S,Sk,q_start,causal", [(F32, 96, 96, 0, True), (F32, 40, 104, 64, True), (F32, 50, 70, 0, False),
+                                                      (BF16, 128, 128, 0, True), (BF16, 72, 200, 128, True)])
+def test_cpu_patch_formula_variant_c(gpu_device, dtype, S, Sk, q_start, causal):
+    """The reference's CPU patch (convert_imu1_checkpoint.py:73-89: RMS normaliser with eps 1e-8, NO 1/sqrt(d), so
+    logits are gain*d*cos, up to +-64 at head_dim 64) is the family at (eps, sm_scale) = (1e-8, 1): the HIP kernels with
+    those parameters against `cpu_patch_variant_c`, forward and every gradient, q_start and non-causal included.
+    fp32 at 1e-5.  The logit bound leaves the raw-exponent range, so the bf16 forward takes its running-maximum
+    path; a bf16 logit carries the 2^-9 rounding of both normalised operands times its magnitude, sqrt(d) = 8 times
+    the live module's, so the absolute part of the bf16 tolerance is scaled by 8 after the fp32 kernels have met
+    1e-5 on the same inputs, and so is the relative part (a logit error of 2^-8 * |logit| is a RELATIVE error of exp(logit):
+    up to 8 times the live module's); both norm-wise.  The reference itself runs this formula on the CPU in fp32 only."""
+    D, n = 64, 3
+    x = gen(n, 1, 1, S, Sk, D, dtype, no_gk=True, seed=23)
+    gain = torch.tensor([1.0])
+    Q, K, V, dO = (x[k][:, 0].contiguous() for k in ("q", "k", "v", "d_o"))
+    ref_in = [t.double().requires_grad_(True) for t in (Q, K, V, gain)]
+    O_ref = orc.cpu_patch_variant_c(*ref_in, causal, q_start)
+    O_ref.backward(dO.double())
+    ref = {"y": O_ref.detach(), "dq": ref_in[0].grad, "dk": ref_in[1].grad, "dv": ref_in[2].grad, "dg_q": ref_in[3].grad}
+    eps, sc = orc.family_params("C", D)
+    assert (eps, sc) == (1e-8, 1.0)
+
+    def run(dt):
+        dev_in = [t.to(dt).to(gpu_device).requires_grad_(True) for t in (Q, K, V)] + [gain.to(gpu_device).requires_grad_(True)]
+        out = QKNormFlashAttnFunc.apply(*dev_in, causal, q_start, None, None, None, None, 2.0, None, eps, sc)
+        out.backward(dO.to(dt).to(gpu_device))
+        return {"y": out.detach().cpu(), "dq": dev_in[0].grad.cpu(), "dk": dev_in[1].grad.cpu(), "dv": dev_in[2].grad.cpu(),
+                "dg_q": dev_in[3].grad.cpu()}
+
+    print(f"variant C {dtype} S={S} Sk={Sk} q_start={q_start} causal={causal}", flush=True)
+    # yardstick of the scalar gain's gradient (a sum over d of per-dimension gradients that cancel)
+    dgs = float(orc.attention_backward_autograd(
+        x["q"].double(), x["k"].double(), x["v"].double(), torch.ones(D, dtype=torch.float64), None, x["d_o"].double(),
+        eps=eps, sm_scale=sc, causal=causal, q_start=q_start)["dg_q"].abs().sum())
+
+    def check(got, atol, rtol, what):
+        for name, r in ref.items():
+            g = got[name].double().reshape(r.shape)
+            scale = max(float(r.abs().max()), dgs) if name == "dg_q" else float(r.abs().max())
+            err = float((g - r).abs().max())
+            print(f"  {what} {name}: max abs err {err:.2e} (largest entry {float(r.abs().max()):.2e})", flush=True)
+            assert err <= atol + rtol * scale, f"{what} {name}: max abs err {err:.3e} > {atol + rtol * scale:.3e}"
+
+    # fp32: 1e-5, norm-wise (relative to the tensor's largest entry).  Element-wise 1e-5 is not attainable in fp32
+    # arithmetic here: one fp32 ulp of a logit of magnitude 64 is 7.6e-6, which alone moves exp(logit) by 7.6e-6 relative,
+    # and the gradients sum thousands of such terms against entries of size 20.
+    check(run(F32), 1e-5, 1e-5, "fp32")
+    if dtype == BF16:
+        check(run(BF16), 8 * 2e-2, 8 * 1e-2, "bf16")
+
+
 def test_module_state_dict_and_forward(gpu_device):
     m = SelfDotProductAttnQKNorm(64).to(gpu_device)
     assert list(m.state_dict().keys()) == ["gain"] and m.gain.shape == (1,) and m.gain.dtype == torch.float32
@@ -621,13 +736,14 @@ def _module_and_oracle_weights(device, dtype, d_model, H, Hkv, qknorm, value_res
 
 def _weight_close(got, ref, dtype, name, yardstick=None):
     """Weight gradients are sums over every token: tolerance relative to the largest entry (norm-wise).
-    A scalar parameter's gradient is ONE sum over every element of the layer, so the bf16 rounding noise of
+    A scalar parameter's gradient is ONE sum over every element of the layer, so the rounding noise of
     the summands does not shrink with the (cancelling) total: for those the relative part refers to
-    `yardstick`, the sum of the magnitudes of the partial gradients the scalar is the total of (the fp32
-    cases pin the same gradients tightly)."""
-    tol = {BF16: (2e-2, 1e-2), F32: (2e-4, 2e-4)}[dtype]
+    `yardstick`, the sum of the magnitudes of the partial gradients the scalar is the total of.  The fp32 cases
+    pin the same gradients at 1e-5 of that yardstick (measured: the output projection, computed by torch's fp32 GEMM
+    on both sides, agrees with the fp64 oracle to 5e-6 at matmul precision "highest", the default)."""
+    tol = {BF16: (2e-2, 1e-2), F32: (1e-5, 1e-5)}[dtype]
     err = (got.double() - ref).abs().max()
-    scale = ref.abs().max() if yardstick is None or dtype != BF16 else max(float(ref.abs().max()), yardstick)
+    scale = ref.abs().max() if yardstick is None else max(float(ref.abs().max()), yardstick)
     bound = tol[0] + tol[1] * scale
     assert err <= bound, f"{name}: max abs err {float(err):.3e} > {float(bound):.3e} (ref max {float(ref.abs().max()):.3e})"
 
@@ -664,11 +780,14 @@ def test_mhsa_module_matches_oracle(gpu_device, dtype, H, Hkv, d, S, qknorm, val
     # product
     xd = x.to(gpu_device).requires_grad_(True)
     v1d = None if v1 is None else v1.to(gpu_device).requires_grad_(True)
+    if use_v1:  # a layer that is handed v1 returns no V by default (only the first layer's is ever used)
+        assert m(xd.detach(), v1=v1d.detach())[1] is None
+        m.always_return_values = True
     out, V = m(xd, v1=v1d)
     assert out.shape == (b, S, d_model) and V.shape == (b, Hkv, S, d)
     out.backward(d_out.to(gpu_device))
     torch.cuda.synchronize()
-    tol = dict(atol=2e-2, rtol=1e-2) if dtype == BF16 else dict(atol=2e-4, rtol=2e-4)
+    tol = dict(atol=2e-2, rtol=1e-2) if dtype == BF16 else dict(atol=1e-5, rtol=1e-5)
     assert torch.allclose(out.detach().cpu().double(), ref_out.detach(), **tol), (out.detach().cpu().double() - ref_out.detach()).abs().max()
     ref_V_native = orc.unflatten_heads(ref_V.detach(), H)[:, :: H // Hkv]
     assert torch.allclose(V.detach().cpu().double(), ref_V_native, **tol)
@@ -678,7 +797,7 @@ def test_mhsa_module_matches_oracle(gpu_device, dtype, H, Hkv, d, S, qknorm, val
     # yardsticks of the scalar parameters: the gain as a vector of equal entries gives its per-dimension
     # gradients; alpha1 / alpha2 / scale act through (c1, c2), whose gradients are sums over (batch, kv head)
     yard = {}
-    if dtype == BF16:
+    if True:  # both dtypes: in fp32 the same sums carry fp32 rounding noise of the same structure, at 1e-5
         wv = {n: t.detach().clone().requires_grad_(True) for n, t in w.items()}
         if qknorm:
             wv["sdpa_qknorm.gain"] = w["sdpa_qknorm.gain"].detach().expand(d).clone().requires_grad_(True)
@@ -699,9 +818,58 @@ def test_mhsa_module_matches_oracle(gpu_device, dtype, H, Hkv, d, S, qknorm, val
         _weight_close(p.grad.cpu(), w[n].grad, dtype, n, yard.get(n))
 
 
+def test_mhsa_module_cached_step_takes_the_decode_kernels(gpu_device):
+    """Under no_grad (the reference generates under inference_mode, transformer.py:160) a cached single-token step
+    of the module reaches the split-key decode kernels: its attention output is bit-identical to a direct
+    qknorm_attention call on the same operands without grad (which sets SEGPT_FLAG_DECODE) and NOT to the training
+    kernels' result (same call with an input that requires grad); with grad mode on, the module takes the
+    training kernels."""
+    H, Hkv, d, S0 = 6, 2, 64, 333
+    b, d_model = 2, H * d
+    m, _, _ = _module_and_oracle_weights(gpu_device, BF16, d_model, H, Hkv, True, True, "per-head", seed=21)
+    g = torch.Generator().manual_seed(22)
+    x = torch.randn(b, S0 + 1, d_model, generator=g).to(BF16).to(gpu_device)
+    captured = {}
+    lin = m.out.linear
+    hook = lin.register_forward_hook(lambda mod, inp, out: captured.__setitem__("attn_cat", inp[0].detach().clone()))
+
+    def direct(cache, xt, requires_grad):
+        """The kernel call the module makes for token xt, rebuilt outside it."""
+        proj = m.qkv(xt)
+        q = proj[..., : H * d].unflatten(-1, (H, d)).permute(0, 2, 1, 3)
+        n = torch.rsqrt(m.alpha1**2 + m.alpha2**2 + 1e-8)
+        coef = torch.cat([m.scale * m.alpha1 * n, m.scale * m.alpha2 * n]).float().detach()
+        q = q.detach().requires_grad_(requires_grad)
+        y = qknorm_attention(q, cache.keys, cache.values, m.sdpa_qknorm.gain.detach(), None, v_first=cache.values, vr_coef=coef,
+                             gate_logits=m.attn_gate(xt), gate_scale=2.0, q_start=cache.length - 1, rope_cos=m.rope.cos,
+                             rope_sin=m.rope.sin, rope_q_pos0=cache.length - 1, out_bshd=True)
+        return y.detach().permute(0, 2, 1, 3).reshape(b, 1, H * d)
+
+    with torch.no_grad():
+        cache = KVCache()
+        m(x[:, :S0], kv_cache=cache)
+        m(x[:, S0:], kv_cache=cache)
+        mod_nograd = captured["attn_cat"]
+        dec = direct(cache, x[:, S0:], requires_grad=False)
+    trn = direct(cache, x[:, S0:], requires_grad=True)   # grad mode on and an input that wants a gradient: training kernels
+    cache2 = KVCache()
+    with torch.no_grad():
+        m(x[:, :S0], kv_cache=cache2)
+    m(x[:, S0:], kv_cache=cache2)                         # grad mode on, parameters require grad: training kernels
+    mod_grad = captured["attn_cat"]
+    hook.remove()
+    same = lambda a, c: torch.equal(a.view(torch.int16), c.view(torch.int16))
+    assert same(mod_nograd, dec), "the module's no_grad cached step is not the decode kernels' result"
+    assert same(mod_grad, trn), "the module's cached step with grad mode on is not the training kernels' result"
+    assert not same(dec, trn), "decode and training kernels agree bit for bit here: the test cannot tell them apart"
+    assert torch.allclose(dec.float(), trn.float(), atol=2e-2, rtol=1e-2)
+
+
 def test_mhsa_module_generation_with_cache(gpu_device):
-    """Prefill + single-token steps through KVCache (raw, un-expanded keys; split-key decode kernels under
-    no_grad) reproduce one full causal pass and the oracle's cached run."""
+    """Prefill + single-token steps through KVCache (raw, un-expanded keys; under no_grad the steps run the
+    split-key decode kernels, see test_mhsa_module_cached_step_takes_the_decode_kernels) reproduce one full causal
+    pass and the oracle's cached run; the value tensor handed to later layers is mixed for the new rows only and
+    still equals the full pass's."""
     H, Hkv, d, S0, S = 6, 2, 64, 150, 154
     b, d_model = 2, H * d
     m, w, rope = _module_and_oracle_weights(gpu_device, BF16, d_model, H, Hkv, True, True, "per-head", seed=9)
@@ -816,6 +984,7 @@ def test_mhsa_module_compiles_to_one_graph(gpu_device):
 
     H, Hkv, d, S, b = 6, 2, 64, 192, 2
     m, _, _ = _module_and_oracle_weights(gpu_device, BF16, H * d, H, Hkv, True, True, "per-head", seed=13)
+    m.always_return_values = True  # the layer is handed v1 here and its own V is compared too
     g = torch.Generator().manual_seed(14)
     x = torch.randn(b, S, H * d, generator=g).to(BF16).to(gpu_device)
     v1 = torch.randn(Hkv * b, S, d, generator=g).to(BF16).to(gpu_device)
@@ -837,6 +1006,41 @@ def test_mhsa_module_compiles_to_one_graph(gpu_device):
     for other in (compiled, ckpt):
         for r, o in zip(ref, other):
             assert torch.equal(r, o)
+
+
+def test_mhsa_module_compiles_with_the_default_backend(gpu_device):
+    """`torch.compile(module)` with the DEFAULT backend (inductor), as the reference compiles its model
+    (trainer.py:227-228 `model.compile()`): the attention op stays one opaque call into the HIP library while the
+    code around it is generated; outputs and gradients equal the eager module's within the bf16 tolerance (inductor
+    may fuse and reorder the elementwise code around the GEMMs, so bit equality is not asked for).  Skipped, with the
+    reason, where inductor's own toolchain cannot run on the box."""
+    H, Hkv, d, S, b = 6, 2, 64, 192, 2
+    m, _, _ = _module_and_oracle_weights(gpu_device, BF16, H * d, H, Hkv, True, True, "per-head", seed=31)
+    g = torch.Generator().manual_seed(32)
+    x = torch.randn(b, S, H * d, generator=g).to(BF16).to(gpu_device)
+    d_out = torch.randn(b, S, H * d, generator=g).to(BF16).to(gpu_device)
+
+    def run(fn):
+        m.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_(True)
+        out, V = fn(xi)
+        out.backward(d_out)
+        torch.cuda.synchronize()
+        return [out.detach().float(), V.detach().float(), xi.grad.float()] + [p.grad.float().clone() for p in m.parameters()]
+
+    eager = run(m)
+    try:
+        compiled_m = torch.compile(m)  # default backend
+        comp = run(compiled_m)
+    except Exception as e:  # inductor needs a working triton / C++ toolchain at run time
+        name = type(e).__name__
+        if any(k in (name + str(e)) for k in ("BackendCompilerFailed", "InductorError", "triton", "Triton", "CppCompileError", "compiler")):
+            pytest.skip(f"inductor cannot compile on this box: {name}: {str(e)[:300]}")
+        raise
+    for a, c in zip(eager, comp):
+        scale = float(a.abs().max())
+        assert torch.allclose(c, a, atol=2e-2 + 1e-2 * scale * 0, rtol=1e-2) or float((c - a).abs().max()) <= 2e-2 + 1e-2 * scale, \
+            f"compiled vs eager: max abs diff {float((c - a).abs().max()):.3e} (scale {scale:.3e})"
 
 
 def test_dropin_with_every_trailing_positional_equals_canonical_call(gpu_device):
