@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SEGPT_ABI_VERSION 1
+#define SEGPT_ABI_VERSION 2
 
 /* element type of q/k/v/o/gate and their gradients */
 #define SEGPT_DTYPE_BF16 0 /* MFMA path: D in {64, 128}                       */
@@ -58,6 +58,10 @@ extern "C" {
 #define SEGPT_E_ALIGN -10      /* a base pointer is not 16-byte aligned                     */
 #define SEGPT_E_ROPE -12       /* rope tables: one NULL, misaligned, or too short for the positions */
 #define SEGPT_E_STAGE -11      /* unknown stage passed to segpt_attn_bwd_stage              */
+#define SEGPT_E_SCRATCH_LIMIT -13 /* segpt_attn_fwd_noalloc: shape needs more than SEGPT_NOALLOC_SCRATCH_BYTES */
+
+/* size of the library-owned device scratch behind segpt_attn_fwd_noalloc (per GPU, held for the process lifetime) */
+#define SEGPT_NOALLOC_SCRATCH_BYTES (16u << 20)
 
 /* segpt_attn_params.flags */
 #define SEGPT_FLAG_KV_PREPARED 1 /* kv_workspace already holds what the key/value pre-pass writes for these k, v,
@@ -200,6 +204,17 @@ int segpt_attn_bwd_stage(const segpt_attn_params* p, int stage, void* stream);
 /* The same for the forward: segpt_attn_fwd(p, s) is stages SEGPT_FWD_STAGE_PRE, SEGPT_FWD_STAGE_ATTN in this
  * order.  No counterpart in the reference (its forward is the single kernel triton_flash_attn_qknorm.py:22-115). */
 int segpt_attn_fwd_stage(const segpt_attn_params* p, int stage, void* stream);
+
+/* segpt_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands and results as
+ * segpt_attn_fwd, except that p->kv_workspace / kv_workspace_bytes are ignored: the key/value scratch (normalised
+ * keys and mixed values, or the split-key partial results of a SEGPT_FLAG_DECODE call) is a fixed
+ * SEGPT_NOALLOC_SCRATCH_BYTES array inside the library's device image.  The call allocates and frees nothing;
+ * a shape whose segpt_attn_workspace_bytes(p, SEGPT_WS_KV) exceeds the array returns SEGPT_E_SCRATCH_LIMIT
+ * before any launch.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (different
+ * streams or threads) race, and no later call may rely on its contents (SEGPT_FLAG_KV_PREPARED is ignored here, and
+ * a backward must run its own key/value pre-pass on a caller-owned kv_workspace). */
+int segpt_attn_fwd_noalloc(const segpt_attn_params* p, void* stream);
 
 #ifdef __cplusplus
 }

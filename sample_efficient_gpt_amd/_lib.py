@@ -12,13 +12,15 @@ import threading
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "libsegpt_attn.so")
 
-SEGPT_ABI_VERSION = 1
+SEGPT_ABI_VERSION = 2
 SEGPT_DTYPE_BF16 = 0
 SEGPT_DTYPE_FP32 = 1
 SEGPT_FLAG_KV_PREPARED = 1
 SEGPT_FLAG_RUNNING_MAX = 2
 SEGPT_FLAG_DECODE = 4
 SEGPT_FLAG_NO_NORM = 8
+SEGPT_E_SCRATCH_LIMIT = -13
+SEGPT_NOALLOC_SCRATCH_BYTES = 16 << 20
 SEGPT_WS_KV = 0
 SEGPT_WS_BWD = 1
 FWD_STAGES = ("pre", "attn")  # SEGPT_FWD_STAGE_* = index
@@ -32,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "segpt_attn_bwd",
     "segpt_attn_bwd_stage",
     "segpt_attn_fwd_stage",
+    "segpt_attn_fwd_noalloc",
 )
 
 
@@ -109,6 +112,8 @@ def load():
         lib.segpt_attn_bwd_stage.argtypes = [C.POINTER(AttnParams), C.c_int, C.c_void_p]
         lib.segpt_attn_fwd_stage.restype = C.c_int
         lib.segpt_attn_fwd_stage.argtypes = [C.POINTER(AttnParams), C.c_int, C.c_void_p]
+        lib.segpt_attn_fwd_noalloc.restype = C.c_int
+        lib.segpt_attn_fwd_noalloc.argtypes = [C.POINTER(AttnParams), C.c_void_p]
         ver = lib.segpt_abi_version()
         if ver != SEGPT_ABI_VERSION:
             raise RuntimeError(f"libsegpt_attn.so ABI version {ver}, binding expects {SEGPT_ABI_VERSION}")

@@ -1,6 +1,13 @@
 // C ABI of libsegpt_attn.so: argument validation, workspace carve-up and dispatch.
 // No device memory is allocated or freed here; nothing synchronises.
+#include <mutex>
+
 #include "common.hpp"
+
+// Scratch of segpt_attn_fwd_noalloc(): lives in the library's device image, one copy per GPU the library runs on,
+// held until the process ends.  In host code this name is only a handle for hipGetSymbolAddress(); kernels and
+// copies get the per-device address looked up below.
+static __device__ __align__(256) unsigned char scratch[SEGPT_NOALLOC_SCRATCH_BYTES];
 
 namespace segpt {
 
@@ -198,6 +205,7 @@ const char* segpt_strerror(int code) {
     case SEGPT_E_ALIGN: return "a base pointer is not 16-byte aligned (workspace: 256-byte)";
     case SEGPT_E_ROPE: return "rope tables: both or neither, 16-byte aligned, rope_len >= position + rows";
     case SEGPT_E_STAGE: return "unknown stage (expected SEGPT_FWD_STAGE_* / SEGPT_BWD_STAGE_*)";
+    case SEGPT_E_SCRATCH_LIMIT: return "segpt_attn_fwd_noalloc: the key/value scratch this shape needs exceeds SEGPT_NOALLOC_SCRATCH_BYTES";
     default: return code > 0 ? "HIP runtime error raised by a kernel launch" : "unknown segpt error code";
   }
 }
@@ -236,6 +244,49 @@ static int fwd_stage_impl(const segpt_attn_params* p, int stage_lo, int stage_hi
 
 int segpt_attn_fwd(const segpt_attn_params* p, void* stream) {
   return fwd_stage_impl(p, SEGPT_FWD_STAGE_PRE, SEGPT_FWD_STAGE_ATTN, stream);
+}
+
+// Device address of `scratch` on the current device, looked up once per device (first call there).
+static int noalloc_scratch_ptr(void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* ptrs[kMaxDevices] = {};
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return (int)hipErrorInvalidSymbol;
+    ptrs[dev] = ptr;
+  }
+  *out = ptrs[dev];
+  return 0;
+}
+
+int segpt_attn_fwd_noalloc(const segpt_attn_params* p, void* stream) {
+  if (!p) return SEGPT_E_NULL;
+  if (p->struct_bytes != sizeof(segpt_attn_params)) return SEGPT_E_STRUCT;
+  segpt_attn_params q = *p;
+  q.kv_workspace = nullptr;
+  q.kv_workspace_bytes = 0;
+  q.flags &= ~SEGPT_FLAG_KV_PREPARED;  // the scratch is shared by every call on this GPU: never assume its contents
+  if (q.dtype == SEGPT_DTYPE_BF16) {
+    if (segpt_attn_workspace_bytes(&q, SEGPT_WS_KV) > (size_t)SEGPT_NOALLOC_SCRATCH_BYTES) return SEGPT_E_SCRATCH_LIMIT;
+    // argument errors first (they need no device): validate against a stand-in address, then look the real one up
+    q.kv_workspace = reinterpret_cast<void*>(uintptr_t{256});
+    q.kv_workspace_bytes = SEGPT_NOALLOC_SCRATCH_BYTES;
+    int rc = check_common(&q);
+    if (!rc) rc = check_t4_out(q.o, q, q.H, q.Sq);
+    if (rc) return rc;
+    void* ptr = nullptr;
+    if ((rc = noalloc_scratch_ptr(&ptr))) return rc;
+    q.kv_workspace = ptr;
+  }
+  return fwd_stage_impl(&q, SEGPT_FWD_STAGE_PRE, SEGPT_FWD_STAGE_ATTN, stream);
 }
 
 int segpt_attn_fwd_stage(const segpt_attn_params* p, int stage, void* stream) {

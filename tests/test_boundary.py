@@ -102,6 +102,12 @@ def test_argument_errors_are_reported_before_any_launch(lib):
     p = _valid_params(); p.workspace, p.workspace_bytes = 0x20000, 1 << 30
     p.dk = _lib.Tensor4(0x10000, 2 * 128 * 64, 64, 64)  # heads interleaved at the row pitch: rows collide
     assert lib.segpt_attn_bwd(p, None) == -6
+    # the entry point with the library's own scratch validates the same way and needs no kv_workspace
+    assert lib.segpt_attn_fwd_noalloc(None, None) == -1
+    p = _valid_params(); p.kv_workspace, p.kv_workspace_bytes = None, 0; p.q.stride_s = 60
+    assert lib.segpt_attn_fwd_noalloc(p, None) == -6
+    p = _valid_params(); p.B, p.Sk = 4096, 4096  # 4096 * 2 * 4096 * 64 * 2 B of normalised keys
+    assert lib.segpt_attn_fwd_noalloc(p, None) == _lib.SEGPT_E_SCRATCH_LIMIT
     p = _valid_params(); p.q_start = -1
     assert lib.segpt_attn_fwd(p, None) == -9
     p = _valid_params(); p.v.ptr = 0x10004
