@@ -10,7 +10,8 @@ key normalisation runs once per step).  Prints ONE JSON line:
              convention; norm/softmax/gate/mix work and recomputation are not credited)
   roofline   the slowest kernel of the step: its credited FLOPs / its average duration, measured
              with HIP events recorded on the launch stream between the stages while the same K steps
-             are replayed stage by stage (segpt_attn_fwd_stage / segpt_attn_bwd_stage), vs the MI355X dense bf16 MFMA peak
+             are replayed stage by stage (segpt_attn_fwd_stage / segpt_attn_bwd_stage; the cost of an empty
+             event pair, measured in the same pass, is subtracted), vs the MI355X dense bf16 MFMA peak
   cpu_baseline  the CPU restatement of the reference's live path (fp32 RMS-normalise ->
              scaled_dot_product_attention(is_causal) -> autograd backward) timed on this host on a
              bounded sample of the same workload
@@ -74,6 +75,43 @@ def cpu_baseline(c, batches: int, budget_s: float = 12.0):
     }
 
 
+def _read_sclk_mhz():
+    """Current shader clock in MHz from sysfs (the level marked '*' in pp_dpm_sclk), or None."""
+    import glob
+    import re
+
+    best = None
+    for path in glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"):
+        try:
+            for line in open(path):
+                if "*" in line:
+                    m = re.search(r"(\d+)\s*M[Hh]z", line)
+                    if m:
+                        best = max(best or 0, int(m.group(1)))
+        except OSError:
+            pass
+    return best
+
+
+def sample_sclk_under_load(step, seconds=0.25):
+    """Median shader clock while the same step loops on the GPU (sampled from a host thread between enqueues)."""
+    import torch
+
+    samples = []
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            step()
+        v = _read_sclk_mhz()
+        if v:
+            samples.append(v)
+        torch.cuda.synchronize()
+    if not samples:
+        return None
+    samples.sort()
+    return samples[len(samples) // 2]
+
+
 def decode_bench(args):
     """One generation step: q [B,18,1,64] against k, v [B,6,Sk,64] (bf16), keys normalised on the fly."""
     import torch
@@ -120,6 +158,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (default: also a HIP-graph replay of the same step)")
     ap.add_argument("--cpu-batches", type=int, default=2)
+    ap.add_argument("--prewarm", type=float, default=0.3,
+                    help="seconds of the same step run UNTIMED before the --warmup steps, so that the shader clock has "
+                         "ramped from its idle level whatever power state the box was in (reported as `prewarm_s`; "
+                         "0 disables it)")
     ap.add_argument("--decode-keys", type=int, default=0,
                     help="instead of a training config: one generation step (1 new token per sequence, IMU-1 heads) "
                          "against a cache of this many keys, through the split-key decode kernels; reports K+V GB/s")
@@ -164,6 +206,7 @@ def main():
             for s in (1, 2, 3):  # stage 0 (the key/value pre-pass) is skipped: kv_prepared
                 plan.backward_stage(s, kv_prepared=True)
                 events[2 + s].record()
+        events[len(names) + 1].record()  # nothing between the last two events: what an event pair alone costs
 
     if args.copy_mib > 0:
         src = torch.empty(args.copy_mib << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -171,6 +214,15 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    # untimed pre-warm: a fresh box idles at ~1.46 GHz and takes a few milliseconds of load to reach its working
+    # clock; W = 5 warm-up steps are 2 ms.  Not part of `warmup` or of the timed region.
+    prewarm_steps = 0
+    tw = time.perf_counter()
+    while time.perf_counter() - tw < args.prewarm:
+        for _ in range(20):
+            step_plain()
+        torch.cuda.synchronize()
+        prewarm_steps += 20
     for _ in range(args.warmup):
         step_plain()
     # ---- timed region: exactly K steps through segpt_attn_fwd + segpt_attn_bwd
@@ -218,16 +270,20 @@ def main():
     # ---- per-kernel durations: the same K steps replayed stage by stage with HIP events recorded on the
     # launch stream between the stages (events in the queue cost a few us per step, which is why the
     # headline number above comes from the uninstrumented loop)
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)] for _ in range(args.steps)]
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 2)] for _ in range(args.steps)]
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     for i in range(args.steps):
         step_staged(evs[i])
     torch.cuda.synchronize()
     ms_staged = (time.perf_counter() - t1) / args.steps * 1e3
-    kern_ms = {n: sum(e[j].elapsed_time(e[j + 1]) for e in evs) / args.steps for j, n in enumerate(names)}
+    # an interval between two events holds the kernel plus the events' own cost in the queue: measured on a pair with
+    # nothing in between (about 4 us) and subtracted, so that the figures agree with the profiler's kernel durations
+    pair_ms = sum(e[len(names)].elapsed_time(e[len(names) + 1]) for e in evs) / args.steps
+    kern_ms = {n: max(sum(e[j].elapsed_time(e[j + 1]) for e in evs) / args.steps - pair_ms, 1e-6) for j, n in enumerate(names)}
     step_ms = sorted(e[0].elapsed_time(e[len(names)]) for e in evs)  # first to last event of each replayed step
 
+    sclk = sample_sclk_under_load(step_plain)
     unit = c.B * c.H * c.S * c.S * c.D  # one causal S x S x D contraction, in FLOPs
     credited = {"fwd": 2 * unit, "bwd_dkdv": 4 * unit, "bwd_dq": 1 * unit}  # dq's recomputed S and dP are not credited
     total_flops = c.flops()
@@ -269,6 +325,9 @@ def main():
             "algorithmic_flops_per_step": total_flops,
         },
         "pct_of_bf16_mfma_peak": round(100 * value / MI355X_BF16_DENSE_TFLOPS, 2),
+        "prewarm_s": args.prewarm,
+        "prewarm_steps": prewarm_steps,
+        "sclk_mhz_under_load": sclk,
         "launch_mode": launch_mode,
         "ms_per_step_eager": round(ms_eager, 5),
         "ms_per_step_graph": None if ms_graph is None else round(ms_graph, 5),
@@ -282,10 +341,12 @@ def main():
             "peak": MI355X_BF16_DENSE_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / MI355X_BF16_DENSE_TFLOPS, 4),
+            "sclk_mhz_under_load": sclk,  # the peak assumes 2400 MHz
             "traffic": PMC_TRAFFIC_BYTES_CFG3.get(dom) if args.cfg == 3 else None,
             "credited_flops_per_launch": credited[dom],
             "avg_launch_ms": round(kern_ms[dom], 5),
-            "timing": "HIP events between the stages, second pass over the same K steps",
+            "timing": "HIP events between the stages, second pass over the same K steps, minus the cost of an empty event pair",
+            "event_pair_overhead_ms": round(pair_ms, 5),
         },
         "kernels": kernels,
     }
