@@ -155,6 +155,10 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--cfg", type=int, default=3, help="benchmark configuration (3 = IMU-1 shape fwd+bwd, the headline)")
+    ap.add_argument("--seq-len", type=int, default=0,
+                    help="run the chosen config at this sequence length instead of its own (a side measurement, e.g. the "
+                         "reference's training contexts 768-1152; the workload string says so, the headline stays cfg 3)")
+    ap.add_argument("--batch", type=int, default=0, help="likewise for the batch size")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (default: also a HIP-graph replay of the same step)")
     ap.add_argument("--cpu-batches", type=int, default=2)
@@ -183,6 +187,11 @@ def main():
     if args.decode_keys > 0:
         return decode_bench(args)
     c = CONFIGS[args.cfg]
+    if args.seq_len > 0:
+        c = c.scaled(S=args.seq_len)
+    if args.batch > 0:
+        c = c.scaled(B=args.batch)
+    resized = args.seq_len > 0 or args.batch > 0
     if c.dtype != torch.bfloat16 and args.cfg != 1:
         raise SystemExit("unsupported config")
     dev = torch.device("cuda:0")
@@ -306,7 +315,8 @@ def main():
         kernels[n] = k
 
     out = {
-        "metric": "attention fwd+bwd TFLOP/s at IMU-1 shape, 1 GPU" if args.cfg == 3 else f"attention TFLOP/s, cfg {args.cfg}",
+        "metric": "attention fwd+bwd TFLOP/s at IMU-1 shape, 1 GPU" if args.cfg == 3 and not resized
+                  else f"attention TFLOP/s, cfg {args.cfg}" + (" resized" if resized else ""),
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -342,7 +352,7 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(achieved / MI355X_BF16_DENSE_TFLOPS, 4),
             "sclk_mhz_under_load": sclk,  # the peak assumes 2400 MHz
-            "traffic": PMC_TRAFFIC_BYTES_CFG3.get(dom) if args.cfg == 3 else None,
+            "traffic": PMC_TRAFFIC_BYTES_CFG3.get(dom) if args.cfg == 3 and not resized else None,
             "credited_flops_per_launch": credited[dom],
             "avg_launch_ms": round(kern_ms[dom], 5),
             "timing": "HIP events between the stages, second pass over the same K steps, minus the cost of an empty event pair",

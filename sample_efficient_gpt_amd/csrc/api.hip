@@ -12,15 +12,17 @@ static __device__ __align__(256) unsigned char scratch[SEGPT_NOALLOC_SCRATCH_BYT
 namespace segpt {
 
 int f32_rows_per_block();
-int bf16_dq_rows_per_block(int D);
-int bf16_dkdv_rows_per_block(int D);
+int bf16_dq_grid(const segpt_attn_params& p);
+int bf16_dkdv_grid(const segpt_attn_params& p);
 
 int dq_blocks(const segpt_attn_params& p) {
-  const int rows = p.dtype == SEGPT_DTYPE_FP32 ? f32_rows_per_block() : bf16_dq_rows_per_block(p.D);
+  if (p.dtype != SEGPT_DTYPE_FP32) return bf16_dq_grid(p);
+  const int rows = f32_rows_per_block();
   return ((p.Sq + rows - 1) / rows) * p.H * p.B;
 }
 int dkdv_blocks(const segpt_attn_params& p) {
-  const int rows = p.dtype == SEGPT_DTYPE_FP32 ? f32_rows_per_block() : bf16_dkdv_rows_per_block(p.D);
+  if (p.dtype != SEGPT_DTYPE_FP32) return bf16_dkdv_grid(p);
+  const int rows = f32_rows_per_block();
   return ((p.Sk + rows - 1) / rows) * p.Hkv * p.B;
 }
 

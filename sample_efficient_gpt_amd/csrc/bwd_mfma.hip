@@ -27,6 +27,20 @@ namespace {
 
 constexpr int kBwdRows = 4 * 32;  // rows (queries for dQ, keys for dK/dV) owned by a workgroup
 
+#ifndef SEGPT_DKDV_PIN_ALL
+#define SEGPT_DKDV_PIN_ALL true
+#endif
+// The dK/dV launch pins (batch, kv head) pairs to XCDs only when ALL of them can be pinned: with a spread remainder it
+// was measured 13 % slower at B*Hkv = 12, S = 8192 (where forward and dQ gain 2-4 % from pinning 8 of the 12).
+constexpr bool kDkdvPinOnlyIfAll = SEGPT_DKDV_PIN_ALL;
+__host__ __device__ inline int dkdv_pinned(const segpt_attn_params& p) {
+#ifdef SEGPT_DKDV_NEVER_PIN
+  return 0;
+#else
+  return wg_pinned_pairs(p.B, p.Hkv, kDkdvPinOnlyIfAll);
+#endif
+}
+
 constexpr int kStages = 4;  // LDS ring of streamed stages (two tiles each): tile t lives in stage t % 4
 
 // ============================================================================================ dQ
@@ -59,7 +73,11 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   const int ln = lane & 31, hh = lane >> 5;
   const int rep = p.H / p.Hkv;
   const int n_qt = (p.Sq + BQ - 1) / BQ;
-  const WgCoord wg = decode_wg(blockIdx.x, n_qt, p.B, p.Hkv, rep);
+  const WgCoord wg = decode_wg(blockIdx.x, n_qt, p.B, p.Hkv, rep, wg_pinned_pairs(p.B, p.Hkv, false));
+  if (!wg.valid) {  // idle padding workgroup: its row of the scale-gradient partials must still read as zero
+    if (tid < D) a.dg_part[(int64_t)blockIdx.x * D + tid] = 0.f;
+    return;
+  }
   const int b = wg.b, g = wg.g, h = wg.g * rep + wg.hh;
   const int q0 = wg.tile * BQ;
   const int qw0 = q0 + wave * 32;
@@ -334,7 +352,11 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     return;
   }
   const int bid = blockIdx.x - 1;  // still a fixed rotation of the hardware's round-robin over the XCDs
-  WgCoord wg = decode_wg(bid, n_kvt, p.B, p.Hkv, 1);
+  WgCoord wg = decode_wg(bid, n_kvt, p.B, p.Hkv, 1, dkdv_pinned(p));
+  if (!wg.valid) {  // idle padding workgroup: its (dc1, dc2) partial must still read as zero
+    if (tid < 2) a.dcoef_part[(int64_t)bid * 2 + tid] = 0.f;
+    return;
+  }
   wg.tile = n_kvt - 1 - wg.tile;  // early key tiles see the most queries: issue them first
   const int b = wg.b, g = wg.g;
   const int k0 = wg.tile * BKV;
@@ -566,7 +588,7 @@ template <int D>
 int launch_dkdv_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
   const int n_kvt = (p.Sk + kBwdRows - 1) / kBwdRows;
-  hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D>), dim3((unsigned)(n_kvt * p.Hkv * p.B + 1)), dim3(kThreadsM), 0, st, a);
+  hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D>), dim3((unsigned)(wg_grid(n_kvt, p.B, p.Hkv, 1, dkdv_pinned(p)) + 1)), dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 
@@ -574,14 +596,16 @@ template <int D>
 int launch_dq_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
   const int n_qt = (p.Sq + kBwdRows - 1) / kBwdRows;
-  hipLaunchKernelGGL((bwd_dq_bf16_kernel<D>), dim3((unsigned)(n_qt * p.H * p.B)), dim3(kThreadsM), 0, st, a);
+  hipLaunchKernelGGL((bwd_dq_bf16_kernel<D>), dim3((unsigned)wg_grid(n_qt, p.B, p.Hkv, p.H / p.Hkv, wg_pinned_pairs(p.B, p.Hkv, false))), dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 
 }  // namespace
 
-int bf16_dq_rows_per_block(int) { return kBwdRows; }
-int bf16_dkdv_rows_per_block(int) { return kBwdRows; }
+// workgroups of the two launches (the dK/dV launch has one more, its extra reducing workgroup): the workspace holds one
+// row of partial sums per workgroup, idle padding workgroups included
+int bf16_dq_grid(const segpt_attn_params& p) { return wg_grid((p.Sq + kBwdRows - 1) / kBwdRows, p.B, p.Hkv, p.H / p.Hkv, wg_pinned_pairs(p.B, p.Hkv, false)); }
+int bf16_dkdv_grid(const segpt_attn_params& p) { return wg_grid((p.Sk + kBwdRows - 1) / kBwdRows, p.B, p.Hkv, 1, dkdv_pinned(p)); }
 
 int launch_bwd_dkdv_bf16(const KArgs& a, hipStream_t st) {
   if (a.p.D == 64) return launch_dkdv_t<64>(a, st);

@@ -72,7 +72,8 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
   const int ln = lane & 31, hh = lane >> 5;
   const int rep = p.H / p.Hkv;
   const int n_qt = (p.Sq + BQ - 1) / BQ;
-  const WgCoord wg = decode_wg(blockIdx.x, n_qt, p.B, p.Hkv, rep);
+  const WgCoord wg = decode_wg(blockIdx.x, n_qt, p.B, p.Hkv, rep, wg_pinned_pairs(p.B, p.Hkv, false));
+  if (!wg.valid) return;  // idle padding workgroup (whole workgroup, before any barrier)
   const int b = wg.b, g = wg.g, h = wg.g * rep + wg.hh;
   const int q0 = wg.tile * BQ;
   const int qw0 = q0 + wave * 32 * NQB;  // first query of this wave
@@ -309,7 +310,7 @@ template <int D, bool WIDE>
 int launch_fwd_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
   const int n_qt = (p.Sq + FwdShape<D, WIDE>::kBQ - 1) / FwdShape<D, WIDE>::kBQ;
-  hipLaunchKernelGGL((fwd_bf16_kernel<D, WIDE>), dim3((unsigned)(n_qt * p.H * p.B)), dim3(kThreadsM), 0, st, a);
+  hipLaunchKernelGGL((fwd_bf16_kernel<D, WIDE>), dim3((unsigned)wg_grid(n_qt, p.B, p.Hkv, p.H / p.Hkv, wg_pinned_pairs(p.B, p.Hkv, false))), dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 

@@ -112,6 +112,14 @@ def test_bf16_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
     _case(gpu_device, BF16, B, H, Hkv, Sq, Sk, D, gen_kw=gen_kw, **kw)
 
 
+@pytest.mark.parametrize("S", [768, 896, 1152])
+def test_bf16_reference_training_contexts(gpu_device, S):
+    """The context lengths of the reference's training curriculum (configs/imu1_base.yaml:56,80,105) with the IMU-1 head
+    layout (GQA 3:1, head_dim 64), gate + value residual as the model runs them: 768 and 896 are multiples of the
+    128-row workgroup tile, 1152 is nine tiles (an odd count for the paired 64-row stages)."""
+    _case(gpu_device, BF16, 2, 6, 2, S, S, 64, seed=S, gen_kw={"extras": True}, gate_scale=2.0)
+
+
 def _slice_inputs(c, x, b, g):
     rep = c.H // c.Hkv
     hs = slice(g * rep, (g + 1) * rep)
