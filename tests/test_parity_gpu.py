@@ -103,6 +103,9 @@ def test_fp32_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
         (1, 3, 3, 72, 200, 64, {"q_start": 128}, {}),
         (1, 2, 1, 1, 257, 64, {"q_start": 256}, {}),   # decode step: one query against a 257-key cache
         (8, 2, 1, 128, 128, 64, {}, {}),              # B*Hkv multiple of 8: XCD-pinned workgroup order
+        (3, 6, 3, 300, 300, 64, {}, {}),              # 9 pairs: 8 pinned + 1 spread, 6 left-over workgroups padded to 8
+        (9, 2, 1, 128, 128, 64, {"gate_scale": 2.0}, {"extras": True}),   # 9 pairs, one tile: 2 left-over workgroups + 6 idle
+        (5, 4, 4, 200, 200, 128, {}, {}),             # 20 pairs at head_dim 128: 16 pinned + 4 spread
         (1, 2, 2, 128, 128, 64, {"eps": 1e-8 / 64, "sm_scale": 1 / 64}, {"scalar_gain": True, "no_gk": True}),
         (2, 4, 2, 300, 130, 64, {}, {}),               # causal with more queries than keys: rows >= 130 see every key
         (1, 2, 1, 257, 64, 128, {}, {"extras": True}),
