@@ -1054,6 +1054,28 @@ def test_mhsa_module_compiles_with_the_default_backend(gpu_device):
             f"compiled vs eager: max abs diff {float((c - a).abs().max()):.3e} (scale {scale:.3e})"
 
 
+def test_compiled_module_without_grad_takes_the_inference_route(gpu_device):
+    """Under no_grad the compiled module (aot_eager: the registered op stays one opaque node, its `inference` argument is
+    decided while tracing, in the caller's grad mode) equals the eager module bit for bit, for a prefill-shaped call and
+    for a decode-shaped one (few query rows against many keys: the split-key kernels)."""
+    H, Hkv, d, b = 6, 2, 64, 2
+    m, _, _ = _module_and_oracle_weights(gpu_device, BF16, H * d, H, Hkv, True, True, "per-head", seed=41)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(b, 200, H * d, generator=g).to(BF16).to(gpu_device)
+    cm = torch.compile(m, backend="aot_eager")
+    with torch.no_grad():
+        e_out, e_V = m(x)
+        c_out, c_V = cm(x)
+        assert torch.equal(e_out, c_out) and torch.equal(e_V, c_V)
+        # decode-shaped: one new token against a 333-key cache, through the op directly (the cache object is host state)
+        q = torch.randn(b, H, 1, d, generator=g).to(BF16).to(gpu_device)
+        k = torch.randn(b, Hkv, 333, d, generator=g).to(BF16).to(gpu_device)
+        v = torch.randn(b, Hkv, 333, d, generator=g).to(BF16).to(gpu_device)
+        f = lambda q, k, v: qknorm_attention_op(q, k, v, m.sdpa_qknorm.gain, None, q_start=332)
+        assert torch.equal(f(q, k, v), torch.compile(f, backend="aot_eager", fullgraph=True)(q, k, v))
+        assert torch.equal(f(q, k, v), qknorm_attention(q, k, v, m.sdpa_qknorm.gain, None, q_start=332))
+
+
 def test_dropin_with_every_trailing_positional_equals_canonical_call(gpu_device):
     """The flattened drop-in with k_gain, v_first, vr_coef, gate_logits, gate_scale, n_kv_heads, eps, sm_scale and
     the rope tables against the canonical-layout call on the same data: same kernels, so outputs and every
