@@ -17,7 +17,8 @@
  *     synchronises: work is enqueued on `stream` and the call returns;
  *   - return value: 0 ok; < 0 argument / unsupported-shape error detected before
  *     any launch (SEGPT_E_*); > 0 a hipError_t raised by a launch;
- *   - re-entrant: no mutable global state.
+ *   - re-entrant: no mutable global state (except segpt_attn_fwd_noalloc, whose calls share one device scratch
+ *     array per GPU: see its comment).
  *
  * Mathematics (per batch b, query head h, kv head g = h / (H/Hkv)):
  *   a_i = rsqrt(mean_d q_i^2 + eps)      b_j = rsqrt(mean_d k_j^2 + eps)
