@@ -65,8 +65,12 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   const segpt_attn_params& p = a.p;
   __shared__ __attribute__((aligned(1024))) char lds[kStages * kStageBytes];
   __shared__ __attribute__((aligned(16))) float gsm[D];       // g_q * g_k, read as float4 slices
-  __shared__ __attribute__((aligned(16))) float red4[4 * D];  // per-wave column sums of the dg partial
-  static_assert(kStages * kStageBytes >= 128 * (D + 1) * 4, "LDS reuse for the dg partial");
+  constexpr int kRedStride = D + 4;                 // floats per row of the dg staging area (16-byte aligned rows)
+  constexpr int kColGroups = D / 4;                 // a thread sums 4 adjacent columns ...
+  constexpr int kRowGroups = kThreadsM / kColGroups;  // ... over one of these groups of rows
+  constexpr int kRowsPerGroup = BQ / kRowGroups;
+  __shared__ __attribute__((aligned(16))) float red4[kRowGroups * D];  // per-row-group column sums of the dg partial
+  static_assert(kStages * kStageBytes >= BQ * kRedStride * 4, "LDS reuse for the dg partial");
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: everything derived from it stays scalar
@@ -170,6 +174,14 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
       }
     }
   }
+  // the query row once more, in the layout of the epilogue's C tiles: requested here, where its latency
+  // is hidden, and carried through the loop as packed pairs
+  u32x2 qct[MB][4];
+  {
+    const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row_c);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) load_ct_block_raw(qp, mb, hh, qct[mb]);
+  }
   // row statistics as MFMA C operands (every register of a lane belongs to the lane's query); the dK/dV
   // kernel reads the same two numbers per row from the workspace
   const float nlse2 = -p.lse[ridx] * kLog2e;
@@ -265,14 +277,14 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   }
 
   // ---- epilogue.  acc = T^T: lane = query, registers = head-dim entries.
-  const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row_c);
   float dot = 0.f;
   float* red = reinterpret_cast<float*>(lds);
   // q in the C-tile layout (rotated like the operand was), then dq = a (u - (a^2/D)(u.q) q) in the rotated frame
   // and back through the transpose of the rotation
   float qv[MB][16];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) load_ct_block(qp, mb, hh, qv[mb]);
+  for (int mb = 0; mb < MB; ++mb) unpack_ct_block(qct[mb], qv[mb]);
+  const float aq = live ? alpha : 0.f;  // padding rows add nothing to the scale gradient
   const float* cosr = nullptr;
   const float* sinr = nullptr;
   if (p.rope_cos) {
@@ -288,14 +300,16 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
       const int d0 = 32 * mb + 8 * c + 4 * hh;
       const float4 g4 = *reinterpret_cast<const float4*>(gsm + d0);
       const float gv[4] = {g4.x, g4.y, g4.z, g4.w};
+      float dgc[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 4 * c + i;
         const float t = acc[mb][r] * p.sm_scale;                 // sm_scale * T
-        red[(wave * 32 + ln) * (D + 1) + d0 + i] = live ? t * alpha * qv[mb][r] : 0.f;  // dg contribution of this row
+        dgc[i] = t * aq * qv[mb][r];                             // dg contribution of this row
         acc[mb][r] = t * gv[i];                                  // u = dL/d(a q)
         dot += acc[mb][r] * qv[mb][r];
       }
+      *reinterpret_cast<float4*>(red + (wave * 32 + ln) * kRedStride + d0) = make_float4(dgc[0], dgc[1], dgc[2], dgc[3]);
     }
   }
   dot = half_sum(dot);
@@ -312,14 +326,23 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   // workgroup partial of dg: column sums over the 128 (wave, lane%32) rows, in two levels so that all
   // 256 threads share the LDS reads (fixed order: deterministic)
   __syncthreads();
-  for (int col = tid & 63; col < D; col += 64) {
-    float t = 0.f;
-#pragma unroll 8
-    for (int x = 0; x < 32; ++x) t += red[(wave * 32 + x) * (D + 1) + col];
-    red4[wave * D + col] = t;
+  {
+    const int cg = tid % kColGroups, rg = tid / kColGroups;
+    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int x = 0; x < kRowsPerGroup; ++x) {
+      const float4 v = *reinterpret_cast<const float4*>(red + (rg * kRowsPerGroup + x) * kRedStride + 4 * cg);
+      t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+    }
+    *reinterpret_cast<float4*>(red4 + rg * D + 4 * cg) = t;
   }
   __syncthreads();
-  if (tid < D) a.dg_part[(int64_t)blockIdx.x * D + tid] = (red4[tid] + red4[D + tid]) + (red4[2 * D + tid] + red4[3 * D + tid]);
+  if (tid < D) {
+    float t = 0.f;
+#pragma unroll
+    for (int x = 0; x < kRowGroups; ++x) t += red4[x * D + tid];
+    a.dg_part[(int64_t)blockIdx.x * D + tid] = t;
+  }
 }
 
 // ============================================================================================ dK, dV

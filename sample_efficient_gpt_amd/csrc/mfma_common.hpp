@@ -278,6 +278,19 @@ __device__ __forceinline__ void load_ct_block(const uint16_t* rowp, int mb, int 
   }
 }
 
+// the same 16 columns kept as packed bf16 pairs (8 registers), for a row that is read early and used late
+__device__ __forceinline__ void load_ct_block_raw(const uint16_t* rowp, int mb, int hh, u32x2 (&out)[4]) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c) out[c] = *reinterpret_cast<const u32x2*>(rowp + 32 * mb + 8 * c + 4 * hh);
+}
+__device__ __forceinline__ void unpack_ct_block(const u32x2 (&w)[4], float (&out)[16]) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    out[4 * c + 0] = bf16lo(w[c][0]); out[4 * c + 1] = bf16hi(w[c][0]);
+    out[4 * c + 2] = bf16lo(w[c][1]); out[4 * c + 3] = bf16hi(w[c][1]);
+  }
+}
+
 __device__ __forceinline__ f32x16 splat16(float x) {
   f32x16 v;
 #pragma unroll
