@@ -101,9 +101,14 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   const uint32_t lds0 = lds_addr_of(lds);
   const int2 src = swz_src<D>(lane, wave);
   const uint32_t wave_dst = lds0 + wave * 1024;
+  const TileLaneOff<D> full_tile = tile_lane_offsets<D>(kstep, vstep, kBK, src.x, src.y);
   auto issue_tile = [&](int jt) {  // tile jt -> stage jt % kStages
-    issue_tile_pair<D>(kbase + (int64_t)jt * kBK * kstep, kstep, vbase + (int64_t)jt * kBK * vstep, vstep,
-                       p.Sk - jt * kBK, wave_dst + (jt % kStages) * kStageBytes, src.x, src.y);
+    const char* ksrc = kbase + (int64_t)jt * kBK * kstep;
+    const char* vsrc = vbase + (int64_t)jt * kBK * vstep;
+    const uint32_t dst = wave_dst + (jt % kStages) * kStageBytes;
+    const int left = p.Sk - jt * kBK;
+    if (left >= kBK) issue_tile_pair<D>(ksrc, vsrc, full_tile, dst);
+    else issue_tile_pair<D>(ksrc, vsrc, tile_lane_offsets<D>(kstep, vstep, left, src.x, src.y), dst);
   };
 
   // start-up tiles first: their latency overlaps the query-row prologue below (vector-memory waits are in
@@ -401,24 +406,51 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   const int2 src = swz_src<D>(lane, wave);
   const bool do_contig = a.do_eff != nullptr;
   const float* const stat_arr = (wave & 1) ? a.delta : a.nlse2;
-  auto issue_tile = [&](int it) {  // streamed tile it -> stage it % kStages
-    const int hq = it / n_vis;
-    const int i0 = (qt_start + it - hq * n_vis) * kBK;
-    const int h = g * rep + hq;
-    const int64_t base = ((int64_t)b * p.H + h) * p.Sq;
-    const char* qsrc = reinterpret_cast<const char*>(a.qhat + (base + i0) * D);
-    const char* dsrc = do_contig ? reinterpret_cast<const char*>(reinterpret_cast<const uint16_t*>(a.do_eff) + (base + i0) * D)
-                                 : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, i0));
-    const uint32_t dstep = do_contig ? (uint32_t)D * 2 : (uint32_t)p.d_o.stride_s * 2;
-    const int stage = it % kStages;
-    issue_tile_pair<D>(qsrc, D * 2, dsrc, dstep, p.Sq - i0, lds0 + stage * kStageBytes + wave * 1024, src.x, src.y);
-    gload_lds4(stat_arr + base + min(i0 + lane, p.Sq - 1), ldl0 + (stage * 128 + (wave & 1) * 64) * 4);
+  const uint32_t dstep = do_contig ? (uint32_t)D * 2 : (uint32_t)p.d_o.stride_s * 2;
+  const TileLaneOff<D> full_tile = tile_lane_offsets<D>(D * 2, dstep, kBK, src.x, src.y);
+  // The stream of (head, query tile) pairs is walked by running pointers kept beside the compute loop's own
+  // counters (three tiles ahead of it): per tile a few scalar additions, per head one address computation.
+  const char* q_it = nullptr;
+  const char* d_it = nullptr;
+  const float* s_it = nullptr;
+  int left_it = 0, iss_h = 0, iss_t = 0, iss_stage = 0;
+  auto set_head = [&](int hq) {
+    const int h = g * rep + hq, i0 = qt_start * kBK;
+    const int64_t row = ((int64_t)b * p.H + h) * p.Sq + i0;
+    q_it = reinterpret_cast<const char*>(a.qhat + row * D);
+    d_it = do_contig ? reinterpret_cast<const char*>(reinterpret_cast<const uint16_t*>(a.do_eff) + row * D)
+                     : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, i0));
+    s_it = stat_arr + row;
+    left_it = p.Sq - i0;
+  };
+  if (n_it > 0) set_head(0);
+  const uint32_t lane4 = lane * 4;
+  auto issue_next = [&]() {
+    const uint32_t dst = lds0 + iss_stage * kStageBytes + wave * 1024;
+    const uint32_t sdst = ldl0 + (iss_stage * 128 + (wave & 1) * 64) * 4;
+    if (left_it >= kBK) {
+      issue_tile_pair<D>(q_it, d_it, full_tile, dst);
+      gload_lds4_so(s_it, lane4, sdst);
+    } else {
+      issue_tile_pair<D>(q_it, d_it, tile_lane_offsets<D>(D * 2, dstep, left_it, src.x, src.y), dst);
+      gload_lds4_so(s_it, (uint32_t)min(lane, left_it - 1) * 4, sdst);
+    }
+    iss_stage = iss_stage == kStages - 1 ? 0 : iss_stage + 1;
+    if (++iss_t == n_vis) {
+      iss_t = 0;
+      if (++iss_h < rep) set_head(iss_h);
+    } else {
+      q_it += kBK * D * 2;
+      d_it += (int64_t)kBK * dstep;
+      s_it += kBK;
+      left_it -= kBK;
+    }
   };
 
   // start-up tiles first: their latency overlaps the loads of the stationary operands below
-  if (n_it > 0) issue_tile(0);
-  if (n_it > 1) issue_tile(1);
-  if (n_it > 2) issue_tile(2);
+  if (n_it > 0) issue_next();
+  if (n_it > 1) issue_next();
+  if (n_it > 2) issue_next();
 
   // stationary B operands: Khat and V' rows of this lane's key
   bf16x8 kreg[KS], vreg[KS];
@@ -524,7 +556,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
       const uint32_t st = st_lane + stage * 512;
       step(masked_c, tr, st, 0, i0, rm, 1);
       step(masked_c, tr, st, 1, i0 + 32, rm_lane + nstage * kStageBytes, 0);
-      if (it + 3 < n_it) { issue_tile(it + 3); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
+      if (it + 3 < n_it) { issue_next(); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
       __syncthreads();
       stage = nstage;
     }

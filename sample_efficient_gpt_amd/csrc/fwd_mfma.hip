@@ -90,9 +90,14 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
   const uint32_t lds0 = lds_addr_of(lds);
   const int2 src = swz_src<D>(lane, wave);
   const uint32_t wave_dst = lds0 + wave * 1024;
+  const TileLaneOff<D> full_tile = tile_lane_offsets<D>(kstep, vstep, kBK, src.x, src.y);
   auto issue_tile = [&](int jt) {  // tile jt -> stage jt % NS
-    issue_tile_pair<D>(kbase + (int64_t)jt * kBK * kstep, kstep, vbase + (int64_t)jt * kBK * vstep, vstep,
-                       p.Sk - jt * kBK, wave_dst + (jt % NS) * kStageBytes, src.x, src.y);
+    const char* ksrc = kbase + (int64_t)jt * kBK * kstep;
+    const char* vsrc = vbase + (int64_t)jt * kBK * vstep;
+    const uint32_t dst = wave_dst + (jt % NS) * kStageBytes;
+    const int left = p.Sk - jt * kBK;
+    if (left >= kBK) issue_tile_pair<D>(ksrc, vsrc, full_tile, dst);
+    else issue_tile_pair<D>(ksrc, vsrc, tile_lane_offsets<D>(kstep, vstep, left, src.x, src.y), dst);
   };
 
   // start-up tiles 0 .. NS-2 first: their latency overlaps the query prologue below (vector-memory waits are

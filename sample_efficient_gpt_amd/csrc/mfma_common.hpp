@@ -110,6 +110,20 @@ __device__ __forceinline__ void gload_lds16(const void* gsrc, uint32_t lds_dst_w
                : "v"(gsrc), "s"(lds_dst_wave_uniform)
                : "memory", "m0");
 }
+// the same load addressed as a wave-uniform base pointer plus a 32-bit byte offset per lane (no 64-bit vector
+// arithmetic per load; the offset can be loop-invariant while the base walks over the tensor)
+__device__ __forceinline__ void gload_lds16_so(const void* base_wave_uniform, uint32_t lane_off, uint32_t lds_dst_wave_uniform) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_off), "s"(base_wave_uniform), "s"(lds_dst_wave_uniform)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void gload_lds4_so(const void* base_wave_uniform, uint32_t lane_off, uint32_t lds_dst_wave_uniform) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+               :
+               : "v"(lane_off), "s"(base_wave_uniform), "s"(lds_dst_wave_uniform)
+               : "memory", "m0");
+}
 __device__ __forceinline__ void gload_lds4(const void* gsrc, uint32_t lds_dst_wave_uniform) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
                :
@@ -298,19 +312,35 @@ __device__ __forceinline__ f32x16 splat16(float x) {
   return v;
 }
 
-// Issue the direct global->LDS loads of two [64, D] bf16 tiles (rows row0..row0+63 of two row-major
-// tensors; rows past nrows re-read the last valid row, callers mask them) into one stage.
-//   src_a/src_b: wave-uniform pointers to row `row0` of each tensor; step_*: bytes between rows
-//   dst: LDS byte address of the stage + wave*1024 (wave-uniform); lane_row / lane_col: from swz_src()
+// Direct global->LDS loads of two [64, D] bf16 tiles (rows row0..row0+63 of two row-major tensors) into one
+// stage.  The lane's byte offsets from row `row0` do not depend on the tile as long as it is full, so they are
+// computed once (rows_left = 64) and a tile then costs no vector arithmetic; a last, partial tile gets its own
+// set, in which rows past rows_left re-read the last valid row (callers mask them).
+//   step_*: bytes between rows; lane_row / lane_col: from swz_src()
 template <int D>
-__device__ __forceinline__ void issue_tile_pair(const char* src_a, uint32_t step_a, const char* src_b, uint32_t step_b,
-                                                int rows_left, uint32_t dst, int lane_row, int lane_col) {
+struct TileLaneOff {
+  uint32_t a[Swz<D>::kPasses], b[Swz<D>::kPasses];
+};
+template <int D>
+__device__ __forceinline__ TileLaneOff<D> tile_lane_offsets(uint32_t step_a, uint32_t step_b, int rows_left, int lane_row, int lane_col) {
   using Z = Swz<D>;
+  TileLaneOff<D> o;
 #pragma unroll
   for (int ps = 0; ps < Z::kPasses; ++ps) {
     const int row = min(lane_row + ps * 4 * Z::kRowsPerInst, rows_left - 1);
-    gload_lds16(src_a + (uint32_t)row * step_a + lane_col, dst + ps * 4096);
-    gload_lds16(src_b + (uint32_t)row * step_b + lane_col, dst + Z::kTileBytes + ps * 4096);
+    o.a[ps] = (uint32_t)row * step_a + lane_col;
+    o.b[ps] = (uint32_t)row * step_b + lane_col;
+  }
+  return o;
+}
+//   src_a/src_b: wave-uniform pointers to row `row0` of each tensor; dst: LDS byte address of the stage + wave*1024
+template <int D>
+__device__ __forceinline__ void issue_tile_pair(const char* src_a, const char* src_b, const TileLaneOff<D>& o, uint32_t dst) {
+  using Z = Swz<D>;
+#pragma unroll
+  for (int ps = 0; ps < Z::kPasses; ++ps) {
+    gload_lds16_so(src_a, o.a[ps], dst + ps * 4096);
+    gload_lds16_so(src_b, o.b[ps], dst + Z::kTileBytes + ps * 4096);
   }
 }
 
