@@ -111,31 +111,67 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     else issue_tile_pair<D>(ksrc, vsrc, tile_lane_offsets<D>(kstep, vstep, left, src.x, src.y), dst);
   };
 
-  // start-up tiles first: their latency overlaps the query-row prologue below (vector-memory waits are in
-  // order, so the prologue's own loads complete after them and nothing stays in flight into the loop)
+  // ---- The workgroup's 128 query / dO / output rows come in as tiles too: read row-per-lane from global memory
+  // every wave-wide load would touch 32 cache lines for 32 bytes each and the prologue would spend its time in
+  // the address path of the vector memory unit; staged through LDS by direct loads they are whole lines, and the
+  // row-major fragment read of a tile is exactly the B-operand layout (lane = row, 8 entries of k-step ks).
+  // Stage 0 takes key tile 0; stages 1..3 hold the q, dO and o blocks until the rows sit in registers, then
+  // key tiles 1 and 2 are requested into stages 1 and 2 and the ring turns as usual.  All of it is in flight at
+  // once, with the row's lse, the gate logit and the scale vector behind it: one memory round trip (vector-memory
+  // waits are in order, and the compiler's own count does not see the direct loads, so its first wait covers
+  // them).  The prologue's results (Qhat, gated dO, -delta, -lse2, dgate) are stored from the epilogue, so no
+  // store is in flight while the loop counts its tile loads.
   issue_tile(0);
+  {
+    const int rows_left = p.Sq - q0;
+    const char* qb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.q, b, h, q0));
+    const char* db = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, q0));
+    const char* yb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.o, b, h, q0));
+    issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, rows_left, src.x, src.y), wave_dst + 1 * kStageBytes);
+    issue_tile_pair<D>(db, db, rowblock_lane_offsets<D>((uint32_t)p.d_o.stride_s * 2, rows_left, src.x, src.y), wave_dst + 2 * kStageBytes);
+    issue_tile_pair<D>(yb, yb, rowblock_lane_offsets<D>((uint32_t)p.o.stride_s * 2, rows_left, src.x, src.y), wave_dst + 3 * kStageBytes);
+  }
+  const float lse_row = p.lse[ridx];
+  // the conditional reads last: the compiler waits for every outstanding load where their branches join
+  float gate_z = 0.f;
+  if (p.gate.ptr)
+    gate_z = bf16_to_f32(reinterpret_cast<const uint16_t*>(p.gate.ptr)[(int64_t)b * p.gate.stride_b + (int64_t)row_c * p.gate.stride_s + (int64_t)h * p.gate.stride_h]);
+  float gval = 0.f;
+  if (tid < D) gval = gprod_at(p, tid);
+  if (tid < D) gsm[tid] = gval;
+  wait_vmcnt<0>();
+  __syncthreads();
+  // rows 32*wave .. 32*wave+31 of the block: half (wave >> 1) of each stage, row block (wave & 1) of that tile
+  u32x4 qraw[KS], dyraw[KS], yraw[KS];
+  u32x2 qct[MB][4];  // the query row once more, in the layout of the epilogue's C tiles (packed pairs)
+  {
+    const uint32_t half = (wave >> 1) * Z::kTileBytes, rb = wave & 1;
+    const uint32_t rm = lds0 + half + swz_off_rm<D>(lane);
+    const uint32_t ct = lds0 + 1 * kStageBytes + half + swz_off_ct<D>(lane) + rb * 32 * Z::kRB;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + 1 * kStageBytes, rb, ks));
+      dyraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + 2 * kStageBytes, rb, ks));
+      yraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + 3 * kStageBytes, rb, ks));
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) qct[mb][c] = lds_read8(ct ^ (uint32_t)((4 * mb + c) << 4));
+  }
+  __syncthreads();  // stages 1 and 2 are free again
   if (n_kt > 1) issue_tile(1);
   if (n_kt > 2) issue_tile(2);
 
   // ---- query-row prologue: alpha, Qhat, delta, gate; B operands stay in registers
-  if (tid < D) gsm[tid] = gprod_at(p, tid);
-  __syncthreads();
   bf16x8 qreg[KS], doreg[KS];
-  float alpha, delta;
+  float alpha, delta, dgate_row = 0.f;
   {
-    const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row_c) + 8 * hh;
-    const uint16_t* yp = row_ptr<uint16_t>(p.o, b, h, row_c) + 8 * hh;
-    const uint16_t* dp = row_ptr<uint16_t>(p.d_o, b, h, row_c) + 8 * hh;
-    u32x4 qraw[KS], dyraw[KS];
     float dl = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      qraw[ks] = *reinterpret_cast<const u32x4*>(qp + 16 * ks);
-      dyraw[ks] = *reinterpret_cast<const u32x4*>(dp + 16 * ks);
-      const u32x4 y = *reinterpret_cast<const u32x4*>(yp + 16 * ks);
+    for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dl += bf16lo(y[i]) * bf16lo(dyraw[ks][i]) + bf16hi(y[i]) * bf16hi(dyraw[ks][i]);
-    }
+      for (int i = 0; i < 4; ++i) dl += bf16lo(yraw[ks][i]) * bf16lo(dyraw[ks][i]) + bf16hi(yraw[ks][i]) * bf16hi(dyraw[ks][i]);
     float qx[KS][8];
     unpack_b_layout<KS>(qraw, qx);
     if (p.rope_cos) {
@@ -153,11 +189,9 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     const float f = alpha * p.sm_scale * kLog2e;
     float gfac = 1.f;
     if (p.gate.ptr) {
-      const float z = bf16_to_f32(reinterpret_cast<const uint16_t*>(p.gate.ptr)[(int64_t)b * p.gate.stride_b + (int64_t)row_c * p.gate.stride_s + (int64_t)h * p.gate.stride_h]);
-      const float sg = 1.0f / (1.0f + __expf(-z));
+      const float sg = 1.0f / (1.0f + __expf(-gate_z));
       gfac = p.gate_scale * sg;
-      if (live && hh == 0)
-        reinterpret_cast<uint16_t*>(p.dgate.ptr)[(int64_t)b * p.dgate.stride_b + (int64_t)row * p.dgate.stride_s + (int64_t)h * p.dgate.stride_h] = f32_to_bf16((1.0f - sg) * delta);
+      dgate_row = (1.0f - sg) * delta;
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -169,28 +203,12 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
       w[2] = pack_bf16x2(qx[ks][4] * f * gb.x, qx[ks][5] * f * gb.y);
       w[3] = pack_bf16x2(qx[ks][6] * f * gb.z, qx[ks][7] * f * gb.w);
       qreg[ks] = as_bf16x8(w);
-      if (live) *reinterpret_cast<u32x4*>(a.qhat + ridx * D + 16 * ks + 8 * hh) = w;
-      if (p.gate.ptr) {
-        const u32x4 e = scale8(dyraw[ks], gfac);
-        doreg[ks] = as_bf16x8(e);
-        if (live) *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(a.do_eff) + ridx * D + 16 * ks + 8 * hh) = e;
-      } else {
-        doreg[ks] = as_bf16x8(dyraw[ks]);
-      }
+      doreg[ks] = as_bf16x8(p.gate.ptr ? scale8(dyraw[ks], gfac) : dyraw[ks]);
     }
-  }
-  // the query row once more, in the layout of the epilogue's C tiles: requested here, where its latency
-  // is hidden, and carried through the loop as packed pairs
-  u32x2 qct[MB][4];
-  {
-    const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row_c);
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) load_ct_block_raw(qp, mb, hh, qct[mb]);
   }
   // row statistics as MFMA C operands (every register of a lane belongs to the lane's query); the dK/dV
   // kernel reads the same two numbers per row from the workspace
-  const float nlse2 = -p.lse[ridx] * kLog2e;
-  if (live && hh == 0) { a.delta[ridx] = -delta; a.nlse2[ridx] = nlse2; }
+  const float nlse2 = -lse_row * kLog2e;
   const f32x16 c_lse = splat16(nlse2);
   const f32x16 c_del = splat16(-delta);
 
@@ -248,10 +266,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     }
   };
 
-  // ---- pipeline start-up: the tile loads that stay in flight across iterations must be the youngest
-  // vector-memory operations of the wave (waits are in-order); here everything has landed.
-  wait_vmcnt<0>();
-  __syncthreads();
+  // ---- pipeline start-up: key tile 0 has landed (first wait above); tiles 1 and 2 are the only vector-memory
+  // operations in flight, which is the state every iteration of the loop leaves behind
   if (n_act > 0) request_rowmajor(rm_lane, 0);
   // leading blocks of this wave that need no mask (every key visible to every query of the wave, inside Sk)
   int n_full = p.Sk / 32;
@@ -281,7 +297,21 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     stage = nstage;
   }
 
-  // ---- epilogue.  acc = T^T: lane = query, registers = head-dim entries.
+  // ---- epilogue.  First what the dK/dV kernel reads of this row: Qhat, the gated dO, -delta, -lse2 (and dgate).
+  if (live) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      *reinterpret_cast<bf16x8*>(a.qhat + ridx * D + 16 * ks + 8 * hh) = qreg[ks];
+      if (p.gate.ptr) *reinterpret_cast<bf16x8*>(reinterpret_cast<uint16_t*>(a.do_eff) + ridx * D + 16 * ks + 8 * hh) = doreg[ks];
+    }
+    if (hh == 0) {
+      a.delta[ridx] = -delta;
+      a.nlse2[ridx] = nlse2;
+      if (p.gate.ptr)
+        reinterpret_cast<uint16_t*>(p.dgate.ptr)[(int64_t)b * p.dgate.stride_b + (int64_t)row * p.dgate.stride_s + (int64_t)h * p.dgate.stride_h] = f32_to_bf16(dgate_row);
+    }
+  }
+  // acc = T^T: lane = query, registers = head-dim entries.
   float dot = 0.f;
   float* red = reinterpret_cast<float*>(lds);
   // q in the C-tile layout (rotated like the operand was), then dq = a (u - (a^2/D)(u.q) q) in the rotated frame

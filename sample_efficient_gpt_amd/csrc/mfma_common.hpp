@@ -333,6 +333,31 @@ __device__ __forceinline__ TileLaneOff<D> tile_lane_offsets(uint32_t step_a, uin
   }
   return o;
 }
+// The same for ONE tensor's 128-row block, staged as the two tiles of a stage (rows 0..63 and 64..127 from the
+// block's first row, of which rows_left >= 1 exist): a = first half, b = second half, both relative to the
+// block's first row, so the block is issued as issue_tile_pair(base, base, offsets, stage).
+template <int D>
+__device__ __forceinline__ TileLaneOff<D> rowblock_lane_offsets(uint32_t step, int rows_left, int lane_row, int lane_col) {
+  using Z = Swz<D>;
+  TileLaneOff<D> o;
+#pragma unroll
+  for (int ps = 0; ps < Z::kPasses; ++ps) {
+    const int r = lane_row + ps * 4 * Z::kRowsPerInst;
+    o.a[ps] = (uint32_t)min(r, rows_left - 1) * step + lane_col;
+    o.b[ps] = (uint32_t)min(r + kBK, rows_left - 1) * step + lane_col;
+  }
+  return o;
+}
+// Per-lane byte offset (within a tile) of the lane's 8 bytes of chunk 0 in the C-tile layout of load_ct_block
+// (lane = row l%32, bytes 8*hh.. of the chunk): chunk c is this offset XOR (c << 4), row block rb adds 32*kRB.
+template <int D>
+__device__ __forceinline__ int swz_off_ct(int lane) {
+  const int ln = lane & 31, hh = lane >> 5;
+  return ln * Swz<D>::kRB + (Swz<D>::f(ln) << 4) + 8 * hh;
+}
+__device__ __forceinline__ u32x2 lds_read8(uint32_t addr) {
+  return *(const __attribute__((address_space(3))) u32x2*)addr;
+}
 //   src_a/src_b: wave-uniform pointers to row `row0` of each tensor; dst: LDS byte address of the stage + wave*1024
 template <int D>
 __device__ __forceinline__ void issue_tile_pair(const char* src_a, const char* src_b, const TileLaneOff<D>& o, uint32_t dst) {
