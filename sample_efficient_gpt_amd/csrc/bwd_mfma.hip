@@ -127,9 +127,9 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     const char* qb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.q, b, h, q0));
     const char* db = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, q0));
     const char* yb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.o, b, h, q0));
-    issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, rows_left, src.x, src.y), wave_dst + 1 * kStageBytes);
-    issue_tile_pair<D>(db, db, rowblock_lane_offsets<D>((uint32_t)p.d_o.stride_s * 2, rows_left, src.x, src.y), wave_dst + 2 * kStageBytes);
-    issue_tile_pair<D>(yb, yb, rowblock_lane_offsets<D>((uint32_t)p.o.stride_s * 2, rows_left, src.x, src.y), wave_dst + 3 * kStageBytes);
+    issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + 1 * kStageBytes);
+    issue_tile_pair<D>(db, db, rowblock_lane_offsets<D>((uint32_t)p.d_o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + 2 * kStageBytes);
+    issue_tile_pair<D>(yb, yb, rowblock_lane_offsets<D>((uint32_t)p.o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + 3 * kStageBytes);
   }
   const float lse_row = p.lse[ridx];
   // the conditional reads last: the compiler waits for every outstanding load where their branches join
@@ -266,8 +266,12 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     }
   };
 
-  // ---- pipeline start-up: key tile 0 has landed (first wait above); tiles 1 and 2 are the only vector-memory
-  // operations in flight, which is the state every iteration of the loop leaves behind
+  // ---- pipeline start-up.  Every iteration of the loop starts with its own tile AND the next one landed (the
+  // second block of a tile already requests the next tile's fragments) and at most one more in flight, so tile 1,
+  // requested after the row blocks had left its stage, must be complete here; the row prologue above ran in
+  // between, so this wait is short.  Tile 2 stays in flight.
+  if (n_kt > 2) wait_vmcnt<kLoadsPerTile>(); else wait_vmcnt<0>();
+  __syncthreads();
   if (n_act > 0) request_rowmajor(rm_lane, 0);
   // leading blocks of this wave that need no mask (every key visible to every query of the wave, inside Sk)
   int n_full = p.Sk / 32;

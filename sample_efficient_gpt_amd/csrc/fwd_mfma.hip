@@ -17,17 +17,16 @@ namespace {
 // Largest |log2-unit logit| the normalised operands can produce: |Qhat.Khat| <= |Qhat| |Khat| with
 // |Khat| <= sqrt(D) and |Qhat| <= sm_scale*log2e*sqrt(D)*max|g_q g_k|.  When it is small the softmax needs
 // no running maximum at all (softmax is shift invariant and exp2 cannot overflow): P = exp2(S2) directly.
-__device__ __forceinline__ float logit_bound(const segpt_attn_params& p, int lane) {
+// Read from the scale vector already in LDS (gsm[d] = sm_scale * log2e * g_q[d] * g_k[d]); 2 % of slack for the
+// bf16 rounding of the operands.
+template <int D>
+__device__ __forceinline__ float logit_bound(const float* gsm, int lane) {
   float gm = 0.f;
-  for (int d = lane; d < p.D; d += 64) {
-    float g = p.gq_numel == 1 ? p.g_q[0] : p.g_q[d];
-    if (p.gk_numel == 1) g *= p.g_k[0];
-    else if (p.gk_numel > 1) g *= p.g_k[d];
-    gm = fmaxf(gm, fabsf(g));
-  }
+#pragma unroll
+  for (int d = lane; d < D; d += 64) gm = fmaxf(gm, fabsf(gsm[d]));
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) gm = fmaxf(gm, __shfl_xor(gm, o, 64));
-  return p.sm_scale * kLog2e * (float)p.D * gm * 1.02f;
+  return (float)D * gm * 1.02f;
 }
 
 constexpr float kNoMaxBound = 64.f;   // |S2| below this: P in [2^-64, 2^64], sums stay far inside fp32 range
@@ -77,7 +76,6 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
   const int b = wg.b, g = wg.g, h = wg.g * rep + wg.hh;
   const int q0 = wg.tile * BQ;
   const int qw0 = q0 + wave * 32 * NQB;  // first query of this wave
-  const bool bounded = !(p.flags & (SEGPT_FLAG_RUNNING_MAX | SEGPT_FLAG_NO_NORM)) && logit_bound(p, lane) <= kNoMaxBound;  // wave-uniform
 
   int kend = p.Sk;
   if (p.causal) kend = min(p.Sk, q0 + BQ + p.q_start);
@@ -100,23 +98,43 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
     else issue_tile_pair<D>(ksrc, vsrc, tile_lane_offsets<D>(kstep, vstep, left, src.x, src.y), dst);
   };
 
-  // start-up tiles 0 .. NS-2 first: their latency overlaps the query prologue below (vector-memory waits are
-  // in order, so the prologue's own loads complete after them and nothing stays in flight into the loop)
+  // ---- start-up.  The workgroup's query rows come in as tiles too (read row-per-lane from global memory, every
+  // wave-wide load would touch 32 cache lines for 32 bytes each; staged through LDS by direct loads they are
+  // whole lines, and the row-major fragment read of a tile is exactly the B-operand layout): they take the last
+  // kQStages stages of the ring, the first kEarlyTiles key tiles (those that fit before them) are requested at the
+  // same time, the scale vector behind them: one memory round trip.  The remaining start-up tiles follow once the
+  // query rows sit in registers (run() below).
+  constexpr int kQStages = BQ / 128;            // 128 rows (two tiles) per stage
+  constexpr int kEarlyTiles = NS - (kQStages > 1 ? kQStages : 1);  // of the NS-1 start-up tiles
+  static_assert(kEarlyTiles >= 2 && kEarlyTiles <= NS - kQStages, "start-up tiles and the query block share the ring");
 #pragma unroll
-  for (int t = 0; t < NS - 1; ++t)
+  for (int t = 0; t < kEarlyTiles; ++t)
     if (t < n_kt) issue_tile(t);
+  {
+    const char* qb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.q, b, h, q0));
+#pragma unroll
+    for (int i = 0; i < kQStages; ++i)
+      issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, 128 * i, p.Sq - q0, src.x, src.y),
+                         wave_dst + (NS - kQStages + i) * kStageBytes);
+  }
 
   // ---- Qhat registers: B operands of S^T, [nb][ks]
-  if (tid < D) gsm[tid] = gprod_at(p, tid) * p.sm_scale * kLog2e;
+  float gval = 0.f;
+  if (tid < D) gval = gprod_at(p, tid) * p.sm_scale * kLog2e;
+  if (tid < D) gsm[tid] = gval;
+  wait_vmcnt<0>();
   __syncthreads();
+  const bool bounded = !(p.flags & (SEGPT_FLAG_RUNNING_MAX | SEGPT_FLAG_NO_NORM)) && logit_bound<D>(gsm, lane) <= kNoMaxBound;  // wave-uniform
   bf16x8 qreg[NQB][KS];
 #pragma unroll
   for (int nb = 0; nb < NQB; ++nb) {
     const int row = min(qw0 + 32 * nb + ln, p.Sq - 1);
-    const uint16_t* qp = row_ptr<uint16_t>(p.q, b, h, row) + 8 * hh;
+    // rows 32*(NQB*wave + nb) .. +31 of the block: 64-row tile (that / 2), row block (that & 1)
+    const int blk = NQB * wave + nb, tile = blk >> 1, rb = blk & 1;
+    const uint32_t rm = lds0 + (NS - kQStages + (tile >> 1)) * kStageBytes + (tile & 1) * Z::kTileBytes + swz_off_rm<D>(lane);
     u32x4 raw[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const u32x4*>(qp + 16 * ks);
+    for (int ks = 0; ks < KS; ++ks) raw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm, rb, ks));
     float x[KS][8];
     unpack_b_layout<KS>(raw, x);
     if (p.rope_cos) {
@@ -247,14 +265,16 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
   if (p.causal) n_full = min(n_full, (qw0 + p.q_start + 1) / 32);
 
   // ---- pipeline.  The tile loads that stay in flight across iterations must be the youngest vector-memory
-  // operations of the wave (waits are in-order): everything is complete at the top of the first iteration.
+  // operations of the wave (waits are in-order): the prologue's wait left nothing else behind.
   // Protocol: at the top of iteration jt tiles jt and jt+1 have landed and tiles jt+2 .. jt+NS-2 are in
   // flight; the stage of tile jt-1 is free (everyone passed the barrier that ended iteration jt-1), so tile
   // jt+NS-1 is requested right away and has a whole iteration to land; the wait at the bottom leaves the
   // youngest NS-3 tiles in flight, i.e. tile jt+2 is complete before the barrier.
   auto run = [&](auto bounded_c) {
-    wait_vmcnt<0>();  // the start-up tiles (requested before the query prologue) have landed
-    __syncthreads();
+    __syncthreads();  // every wave has its query rows in registers: their stages are free
+#pragma unroll
+    for (int t = kEarlyTiles; t < NS - 1; ++t)
+      if (t < n_kt) issue_tile(t);
     if (n_act > 0) request_rowmajor(rm_lane, 0);
     int stage = 0;
     // Two loops instead of a per-block choice inside one: each body is then a single straight-line region

@@ -333,16 +333,16 @@ __device__ __forceinline__ TileLaneOff<D> tile_lane_offsets(uint32_t step_a, uin
   }
   return o;
 }
-// The same for ONE tensor's 128-row block, staged as the two tiles of a stage (rows 0..63 and 64..127 from the
-// block's first row, of which rows_left >= 1 exist): a = first half, b = second half, both relative to the
-// block's first row, so the block is issued as issue_tile_pair(base, base, offsets, stage).
+// The same for 128 rows of ONE tensor, staged as the two tiles of a stage: a = rows row_first .. +63, b = rows
+// row_first+64 .. +127, both as offsets from the tensor block's first row (row 0, of which rows_left >= 1 exist;
+// later rows re-read the last one), so the rows are issued as issue_tile_pair(base, base, offsets, stage).
 template <int D>
-__device__ __forceinline__ TileLaneOff<D> rowblock_lane_offsets(uint32_t step, int rows_left, int lane_row, int lane_col) {
+__device__ __forceinline__ TileLaneOff<D> rowblock_lane_offsets(uint32_t step, int row_first, int rows_left, int lane_row, int lane_col) {
   using Z = Swz<D>;
   TileLaneOff<D> o;
 #pragma unroll
   for (int ps = 0; ps < Z::kPasses; ++ps) {
-    const int r = lane_row + ps * 4 * Z::kRowsPerInst;
+    const int r = row_first + lane_row + ps * 4 * Z::kRowsPerInst;
     o.a[ps] = (uint32_t)min(r, rows_left - 1) * step + lane_col;
     o.b[ps] = (uint32_t)min(r + kBK, rows_left - 1) * step + lane_col;
   }
