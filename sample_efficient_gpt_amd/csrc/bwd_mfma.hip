@@ -425,7 +425,6 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   const int kw0 = k0 + wave * 32;
   const int key = kw0 + ln;
   const int key_c = min(key, p.Sk - 1);
-  const int64_t kidx = ((int64_t)b * p.Hkv + g) * p.Sk + key_c;
 
   const int n_qt = (p.Sq + kBK - 1) / kBK;
   int qt_start = 0;
@@ -481,22 +480,38 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     }
   };
 
-  // start-up tiles first: their latency overlaps the loads of the stationary operands below
+  // ---- start-up: streamed tiles 0 and 1 into stages 0 and 1, and with them the workgroup's 128 Khat and V' rows
+  // as tiles into stages 2 and 3 (whole cache lines by direct loads instead of 16 bytes per lane and row; the
+  // row-major fragment read of a tile is the B-operand layout): one memory round trip.  Once the rows sit in
+  // registers, tile 2 is requested into stage 2 and the ring turns as usual (every iteration needs its own tile and
+  // the next one landed, and leaves one more in flight).
   if (n_it > 0) issue_next();
   if (n_it > 1) issue_next();
-  if (n_it > 2) issue_next();
-
-  // stationary B operands: Khat and V' rows of this lane's key
+  {
+    const int rows_left = p.Sk - k0;
+    const int64_t krow = ((int64_t)b * p.Hkv + g) * p.Sk + k0;
+    const char* kb = reinterpret_cast<const char*>(a.khat + krow * D);
+    const char* vb = a.vmix ? reinterpret_cast<const char*>(a.vmix + krow * D) : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.v, b, g, k0));
+    const uint32_t vstep = a.vmix ? (uint32_t)D * 2 : (uint32_t)p.v.stride_s * 2;
+    const uint32_t wave_dst = lds0 + wave * 1024;
+    issue_tile_pair<D>(kb, kb, rowblock_lane_offsets<D>(D * 2, 0, rows_left, src.x, src.y), wave_dst + 2 * kStageBytes);
+    issue_tile_pair<D>(vb, vb, rowblock_lane_offsets<D>(vstep, 0, rows_left, src.x, src.y), wave_dst + 3 * kStageBytes);
+  }
+  wait_vmcnt<0>();
+  __syncthreads();
+  // stationary B operands: Khat and V' rows of this lane's key (rows 32*wave .. +31 of the block)
   bf16x8 kreg[KS], vreg[KS];
   {
-    const uint16_t* kp = a.khat + kidx * D + 8 * hh;
-    const uint16_t* vp = (a.vmix ? a.vmix + kidx * D : row_ptr<uint16_t>(p.v, b, g, key_c)) + 8 * hh;
+    const uint32_t rm = lds0 + (wave >> 1) * Z::kTileBytes + swz_off_rm<D>(lane);
+    const int rb = wave & 1;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      kreg[ks] = as_bf16x8(*reinterpret_cast<const u32x4*>(kp + 16 * ks));
-      vreg[ks] = as_bf16x8(*reinterpret_cast<const u32x4*>(vp + 16 * ks));
+      kreg[ks] = swz_frag_rm<D>(rm + 2 * kStageBytes, rb, ks);
+      vreg[ks] = swz_frag_rm<D>(rm + 3 * kStageBytes, rb, ks);
     }
   }
+  __syncthreads();  // stages 2 and 3 are free again
+  if (n_it > 2) issue_next();
   f32x16 dvacc[MB], dkacc[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) { dvacc[mb] = splat16(0.f); dkacc[mb] = splat16(0.f); }
@@ -570,9 +585,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     }
   };
 
-  // ---- pipeline start-up (see the dQ kernel)
-  wait_vmcnt<0>();
-  __syncthreads();
+  // ---- pipeline start-up: tiles 0 and 1 have landed (first wait above), tile 2 is in flight
   if (n_it > 0) request_rowmajor(rm_lane, 0);
   // Per head the visible query tiles t = 0 .. n_vis-1 (first query (qt_start + t) * 64) fall into three runs for
   // this wave: [0, t_diag) touch the causal diagonal, [t_diag, t_end) need no mask, [t_end, n_vis) run past Sq.
