@@ -24,8 +24,20 @@ __device__ __forceinline__ float logit_bound(const float* gsm, int lane) {
   float gm = 0.f;
 #pragma unroll
   for (int d = lane; d < D; d += 64) gm = fmaxf(gm, fabsf(gsm[d]));
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) gm = fmaxf(gm, __shfl_xor(gm, o, 64));
+  // wave-wide maximum by six DPP steps (shifts by 1, 2, 4, 8 inside the rows of 16 lanes, then the row maxima
+  // passed on to the next row and the next half): lane 63 ends up with it.  A lane whose source does not exist
+  // keeps its own value.
+  auto step = [](float v, auto ctrl, auto rows) {
+    const int t = __builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), decltype(ctrl)::value, decltype(rows)::value, 0xf, false);
+    return fmaxf(v, __int_as_float(t));
+  };
+  gm = step(gm, IC<0x111>{}, IC<0xf>{});
+  gm = step(gm, IC<0x112>{}, IC<0xf>{});
+  gm = step(gm, IC<0x114>{}, IC<0xf>{});
+  gm = step(gm, IC<0x118>{}, IC<0xf>{});
+  gm = step(gm, IC<0x142>{}, IC<0xa>{});
+  gm = step(gm, IC<0x143>{}, IC<0xc>{});
+  gm = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gm), 63));
   return (float)D * gm * 1.02f;
 }
 

@@ -646,6 +646,32 @@ def test_reference_named_function_defaults_to_the_reference_kernel_formula(gpu_d
     assert float((live.cpu().double() - O_ref.detach()).abs().max()) > 1e-2
 
 
+@pytest.mark.parametrize("D,d_big", [(64, 0), (64, 15), (64, 16), (64, 31), (64, 32), (64, 47), (64, 63),
+                                     (128, 0), (128, 63), (128, 64), (128, 100), (128, 127)])
+def test_bf16_forward_sees_a_single_large_scale_entry(gpu_device, D, d_big):
+    """The bf16 forward drops the running maximum when max_d |g_q g_k| bounds the logits inside the exponent range;
+    that maximum is a wave-wide reduction over the scale vector.  One entry of g_q is made large enough (logits of
+    +-320 in natural units, 2^461 as a raw exponent) that the forward must keep the running maximum, whichever
+    lane and DPP row holds the entry: queries and keys are dominated by that dimension, so a forward that missed
+    the entry would overflow to inf / NaN.  Checked here: the output is finite and every row is a convex
+    combination of value rows (|y| <= max |v|); parity at such logits is the variant-C test's business."""
+    torch.manual_seed(5)
+    B, H, S = 1, 2, 160
+    q = 0.01 * torch.randn(B, H, S, D)
+    k = 0.01 * torch.randn(B, H, S, D)
+    q[..., d_big] = 1.0
+    k[..., d_big] = torch.where(torch.rand(B, H, S) < 0.5, -1.0, 1.0)
+    v = torch.randn(B, H, S, D)
+    g = torch.full((D,), 0.5)
+    g[d_big] = 40.0
+    print(f"large scale entry D={D} at {d_big}", flush=True)
+    dev = lambda t: t.to(BF16).to(gpu_device)
+    y = qknorm_attention(dev(q), dev(k), dev(v), g.to(gpu_device), None, eps=1e-6, sm_scale=D ** -0.5)
+    y = y.float().cpu()
+    assert torch.isfinite(y).all(), "the forward took the no-maximum path with logits outside the exponent range"
+    assert float(y.abs().max()) <= float(v.to(BF16).float().abs().max()) * 1.01
+
+
 @pytest.mark.parametrize("dtype,S,Sk,q_start,causal", [(F32, 96, 96, 0, True), (F32, 40, 104, 64, True), (F32, 50, 70, 0, False),
                                                       (BF16, 128, 128, 0, True), (BF16, 72, 200, 128, True)])
 def test_cpu_patch_formula_variant_c(gpu_device, dtype, S, Sk, q_start, causal):
