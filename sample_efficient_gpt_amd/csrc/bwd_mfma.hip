@@ -530,9 +530,10 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   };
   // one 32-query block (qb = 0/1, compile-time) of the tile whose stage the pointers address;
   // ib = first query of the block; the row-major fragments of the block after it start at next_rm.
-  // MASKED is compile-time so that a whole block is one straight-line scheduling region.
+  // The mask variant is compile-time so that a whole block is one straight-line scheduling region:
+  // 0 none, 1 causal diagonal only (every query of the block exists), 2 diagonal and / or end of the queries.
   auto step = [&](auto masked_c, uint32_t tr, uint32_t st, int qb, int ib, uint32_t next_rm, int next_qb) {
-    constexpr bool MASKED = decltype(masked_c)::value != 0;
+    constexpr int MASK = decltype(masked_c)::value;
     // accumulators of S and dP start from -lse2 / -delta of the 16 query rows their registers map to
     f32x16 s, dpv;
 #pragma unroll
@@ -554,7 +555,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
       dT[mb][1] = swz_frag_tr<D>(tr + Z::kTileBytes, mb, 2 * qb + 1);
       qT[mb][1] = swz_frag_tr<D>(tr, mb, 2 * qb + 1);
     }
-    if (MASKED) {  // block touches the diagonal or the end of the queries
+    if (MASK != 0) {  // block touches the diagonal or the end of the queries
       // register r holds query ib + 4hh + c_r with c_r = 8(r/4) + r%4 a compile-time constant.
       // masked iff key > query + q_start  <=>  c_r < key - q_start - ib - 4hh,   or query >= Sq
       const int t = p.causal ? key - p.q_start - ib - 4 * hh : -1;
@@ -562,7 +563,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int c = 8 * (r >> 2) + (r & 3);
-        if (c < t || c >= u) s[r] = -INFINITY;
+        if (MASK == 1 ? c < t : (c < t || c >= u)) s[r] = -INFINITY;
       }
     }
 #pragma unroll
@@ -587,31 +588,37 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
 
   // ---- pipeline start-up: tiles 0 and 1 have landed (first wait above), tile 2 is in flight
   if (n_it > 0) request_rowmajor(rm_lane, 0);
-  // Per head the visible query tiles t = 0 .. n_vis-1 (first query (qt_start + t) * 64) fall into three runs for
-  // this wave: [0, t_diag) touch the causal diagonal, [t_diag, t_end) need no mask, [t_end, n_vis) run past Sq.
-  // Each run is its own loop so that a loop body holds one variant of the block (whole-block scheduling
-  // regions, no accumulator copies at joins).
+  // Per head the visible query tiles t = 0 .. n_vis-1 (first query (qt_start + t) * 64) fall into runs for this
+  // wave: [0, t_diag) touch the causal diagonal (those before t_full lie inside Sq and need the diagonal test only),
+  // [t_diag, t_end) need no mask, [t_end, n_vis) run past Sq.  Each run is its own loop so that a loop body holds
+  // one variant of the block (whole-block scheduling regions, no accumulator copies at joins).
   int t_diag = 0;
   if (p.causal) t_diag = min(max((max(kw0 + 31 - p.q_start, 0) + kBK - 1) / kBK - qt_start, 0), n_vis);
-  const int t_end = min(max(p.Sq / kBK - qt_start, t_diag), n_vis);
+  const int t_full = min(max(p.Sq / kBK - qt_start, 0), n_vis);  // tiles whose 64 queries all exist
+  const int t_end = max(t_full, t_diag);
   int stage = 0, it = 0;
   auto run_tiles = [&](auto masked_c, int t_lo, int t_hi) {
+    constexpr int MASK = decltype(masked_c)::value;
     for (int t = t_lo; t < t_hi; ++t, ++it) {
       const int nstage = stage == kStages - 1 ? 0 : stage + 1;
       const int i0 = (qt_start + t) * kBK;
       const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
       const uint32_t st = st_lane + stage * 512;
-      step(masked_c, tr, st, 0, i0, rm, 1);
-      step(masked_c, tr, st, 1, i0 + 32, rm_lane + nstage * kStageBytes, 0);
+      // on the diagonal a block whose last query still lies before this wave's first key is masked entirely:
+      // it only passes the fragment request on (wave-uniform, so the barrier below is reached all the same)
+      if (MASK == 1 && kw0 > i0 + 31 + p.q_start) request_rowmajor(rm, 1); else step(masked_c, tr, st, 0, i0, rm, 1);
+      if (MASK == 1 && kw0 > i0 + 63 + p.q_start) request_rowmajor(rm_lane + nstage * kStageBytes, 0);
+      else step(masked_c, tr, st, 1, i0 + 32, rm_lane + nstage * kStageBytes, 0);
       if (it + 3 < n_it) { issue_next(); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
       __syncthreads();
       stage = nstage;
     }
   };
   for (int hq = 0; hq < rep; ++hq) {
-    run_tiles(IC<1>{}, 0, t_diag);
+    run_tiles(IC<1>{}, 0, min(t_diag, t_full));
+    run_tiles(IC<2>{}, min(t_diag, t_full), t_diag);
     run_tiles(IC<0>{}, t_diag, t_end);
-    run_tiles(IC<1>{}, t_end, n_vis);
+    run_tiles(IC<2>{}, t_end, n_vis);
   }
 
   // ---- epilogue: lane = key row, registers = head-dim entries
