@@ -36,7 +36,7 @@ MI355X_HBM_GBS = 8000.0
 # HBM bytes per launch (read + write) at cfg 3, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a plain
 # copy kernel of known size (FETCH_SIZE reads 0.5 of the true bytes on this part, WRITE_SIZE 1.0); profiler numbers,
 # not measured by this script
-PMC_TRAFFIC_BYTES_CFG3 = {"fwd": 120.1e6, "bwd_dq": 266.4e6, "bwd_dkdv": 199.8e6}
+PMC_TRAFFIC_BYTES_CFG3 = {"fwd": 120.1e6, "bwd_dq": 266.3e6, "bwd_dkdv": 208.0e6}
 
 
 def cpu_baseline(c, batches: int, budget_s: float = 12.0):
