@@ -27,19 +27,9 @@ namespace {
 
 constexpr int kBwdRows = 4 * 32;  // rows (queries for dQ, keys for dK/dV) owned by a workgroup
 
-#ifndef SEGPT_DKDV_PIN_ALL
-#define SEGPT_DKDV_PIN_ALL true
-#endif
 // The dK/dV launch pins (batch, kv head) pairs to XCDs only when ALL of them can be pinned: with a spread remainder it
 // was measured 13 % slower at B*Hkv = 12, S = 8192 (where forward and dQ gain 2-4 % from pinning 8 of the 12).
-constexpr bool kDkdvPinOnlyIfAll = SEGPT_DKDV_PIN_ALL;
-__host__ __device__ inline int dkdv_pinned(const segpt_attn_params& p) {
-#ifdef SEGPT_DKDV_NEVER_PIN
-  return 0;
-#else
-  return wg_pinned_pairs(p.B, p.Hkv, kDkdvPinOnlyIfAll);
-#endif
-}
+__host__ __device__ inline int dkdv_pinned(const segpt_attn_params& p) { return wg_pinned_pairs(p.B, p.Hkv, true); }
 
 constexpr int kStages = 4;  // LDS ring of streamed stages (two tiles each): tile t lives in stage t % 4
 
