@@ -21,6 +21,7 @@
 // One workgroup = 4 waves (one per SIMD); several workgroups share a CU so that the softmax-like VALU
 // phase of one overlaps the MFMA phase of another.  Streamed tiles (64 rows) are double-buffered in LDS.
 #include "mfma_common.hpp"
+#include "ring_protocol.hpp"
 
 namespace segpt {
 namespace {
@@ -51,7 +52,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
   constexpr int kStageBytes = 2 * Z::kTileBytes;
-  constexpr int kLoadsPerTile = 2 * Z::kPasses;  // per wave
+  constexpr ring::Protocol R = ring::dq(Z::kPasses);  // the pipeline's numbers: ring_protocol.hpp
+  static_assert(ring::well_formed(R) && R.stages == kStages && R.row_stages == 3 && R.wait_before_loop && !R.issue_at_top, "tile pipeline");
   const segpt_attn_params& p = a.p;
   __shared__ __attribute__((aligned(1024))) char lds[kStages * kStageBytes];
   __shared__ __attribute__((aligned(16))) float gsm[D];       // g_q * g_k, read as float4 slices
@@ -111,15 +113,18 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   // waits are in order, and the compiler's own count does not see the direct loads, so its first wait covers
   // them).  The prologue's results (Qhat, gated dO, -delta, -lse2, dgate) are stored from the epilogue, so no
   // store is in flight while the loop counts its tile loads.
-  issue_tile(0);
+#pragma unroll
+  for (int t = 0; t < R.early_tiles; ++t)
+    if (t < n_kt) issue_tile(t);
+  constexpr int kRowStage = R.row_stage_first;  // q, dO, o blocks in stages kRowStage, +1, +2
   {
     const int rows_left = p.Sq - q0;
     const char* qb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.q, b, h, q0));
     const char* db = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, q0));
     const char* yb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.o, b, h, q0));
-    issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + 1 * kStageBytes);
-    issue_tile_pair<D>(db, db, rowblock_lane_offsets<D>((uint32_t)p.d_o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + 2 * kStageBytes);
-    issue_tile_pair<D>(yb, yb, rowblock_lane_offsets<D>((uint32_t)p.o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + 3 * kStageBytes);
+    issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + kRowStage * kStageBytes);
+    issue_tile_pair<D>(db, db, rowblock_lane_offsets<D>((uint32_t)p.d_o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + (kRowStage + 1) * kStageBytes);
+    issue_tile_pair<D>(yb, yb, rowblock_lane_offsets<D>((uint32_t)p.o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + (kRowStage + 2) * kStageBytes);
   }
   const float lse_row = p.lse[ridx];
   // the conditional reads last: the compiler waits for every outstanding load where their branches join
@@ -137,21 +142,22 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   {
     const uint32_t half = (wave >> 1) * Z::kTileBytes, rb = wave & 1;
     const uint32_t rm = lds0 + half + swz_off_rm<D>(lane);
-    const uint32_t ct = lds0 + 1 * kStageBytes + half + swz_off_ct<D>(lane) + rb * 32 * Z::kRB;
+    const uint32_t ct = lds0 + kRowStage * kStageBytes + half + swz_off_ct<D>(lane) + rb * 32 * Z::kRB;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      qraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + 1 * kStageBytes, rb, ks));
-      dyraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + 2 * kStageBytes, rb, ks));
-      yraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + 3 * kStageBytes, rb, ks));
+      qraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + kRowStage * kStageBytes, rb, ks));
+      dyraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + (kRowStage + 1) * kStageBytes, rb, ks));
+      yraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + (kRowStage + 2) * kStageBytes, rb, ks));
     }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int c = 0; c < 4; ++c) qct[mb][c] = lds_read8(ct ^ (uint32_t)((4 * mb + c) << 4));
   }
-  __syncthreads();  // stages 1 and 2 are free again
-  if (n_kt > 1) issue_tile(1);
-  if (n_kt > 2) issue_tile(2);
+  __syncthreads();  // the borrowed stages are free again
+#pragma unroll
+  for (int t = R.early_tiles; t < R.startup_tiles; ++t)
+    if (t < n_kt) issue_tile(t);
 
   // ---- query-row prologue: alpha, Qhat, delta, gate; B operands stay in registers
   bf16x8 qreg[KS], doreg[KS];
@@ -260,7 +266,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   // second block of a tile already requests the next tile's fragments) and at most one more in flight, so tile 1,
   // requested after the row blocks had left its stage, must be complete here; the row prologue above ran in
   // between, so this wait is short.  Tile 2 stays in flight.
-  if (n_kt > 2) wait_vmcnt<kLoadsPerTile>(); else wait_vmcnt<0>();
+  if (n_kt >= R.startup_tiles) wait_vmcnt<ring::loads_kept_before_loop(R, R.startup_tiles)>(); else wait_vmcnt<0>();
   __syncthreads();
   if (n_act > 0) request_rowmajor(rm_lane, 0);
   // leading blocks of this wave that need no mask (every key visible to every query of the wave, inside Sk)
@@ -277,7 +283,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     step(IC<0>{}, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
     // stage (jt+3) % 4 == (jt-1) % 4 was last read in the previous iteration: refill it, then make sure
     // this wave's part of tile jt+2 (needed from the next iteration's prefetch on) has landed
-    if (jt + 3 < n_kt) { issue_tile(jt + 3); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
+    if (jt + R.issue_ahead < n_kt) { issue_tile(jt + R.issue_ahead); wait_vmcnt<ring::loads_kept_after_iteration(R, true)>(); } else wait_vmcnt<ring::loads_kept_after_iteration(R, false)>();
     __syncthreads();
     stage = nstage;
   }
@@ -286,7 +292,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
     if (2 * jt < n_act) step(IC<1>{}, tr, 0, 64 * jt, rm, 1);
     if (2 * jt + 1 < n_act) step(IC<1>{}, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
-    if (jt + 3 < n_kt) { issue_tile(jt + 3); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
+    if (jt + R.issue_ahead < n_kt) { issue_tile(jt + R.issue_ahead); wait_vmcnt<ring::loads_kept_after_iteration(R, true)>(); } else wait_vmcnt<ring::loads_kept_after_iteration(R, false)>();
     __syncthreads();
     stage = nstage;
   }
@@ -385,7 +391,10 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
   constexpr int kStageBytes = 2 * Z::kTileBytes;
-  constexpr int kLoadsPerTile = 2 * Z::kPasses + 1;  // per wave: the two tiles plus one row-statistics load
+  constexpr ring::Protocol R = ring::dkdv(Z::kPasses);  // the pipeline's numbers: ring_protocol.hpp
+  static_assert(ring::well_formed(R) && R.stages == kStages && R.row_stages == 2 && !R.wait_before_loop && !R.issue_at_top, "tile pipeline");
+  static_assert(R.early_tiles >= ring::kTilesNeededAtLoopStart, "the loop is entered without a further wait");
+  static_assert(R.loads_per_tile == 2 * Z::kPasses + 1, "per wave: the two tiles plus one row-statistics load");
   const segpt_attn_params& p = a.p;
   __shared__ __attribute__((aligned(1024))) char lds[kStages * kStageBytes];
   __shared__ __attribute__((aligned(256))) float ldl[kStages * 128];  // per stage: [0,64) -lse2, [64,128) -delta
@@ -475,8 +484,10 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   // row-major fragment read of a tile is the B-operand layout): one memory round trip.  Once the rows sit in
   // registers, tile 2 is requested into stage 2 and the ring turns as usual (every iteration needs its own tile and
   // the next one landed, and leaves one more in flight).
-  if (n_it > 0) issue_next();
-  if (n_it > 1) issue_next();
+#pragma unroll
+  for (int t = 0; t < R.early_tiles; ++t)
+    if (t < n_it) issue_next();
+  constexpr int kRowStage = R.row_stage_first;  // Khat block in stage kRowStage, V' block in the next
   {
     const int rows_left = p.Sk - k0;
     const int64_t krow = ((int64_t)b * p.Hkv + g) * p.Sk + k0;
@@ -484,8 +495,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     const char* vb = a.vmix ? reinterpret_cast<const char*>(a.vmix + krow * D) : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.v, b, g, k0));
     const uint32_t vstep = a.vmix ? (uint32_t)D * 2 : (uint32_t)p.v.stride_s * 2;
     const uint32_t wave_dst = lds0 + wave * 1024;
-    issue_tile_pair<D>(kb, kb, rowblock_lane_offsets<D>(D * 2, 0, rows_left, src.x, src.y), wave_dst + 2 * kStageBytes);
-    issue_tile_pair<D>(vb, vb, rowblock_lane_offsets<D>(vstep, 0, rows_left, src.x, src.y), wave_dst + 3 * kStageBytes);
+    issue_tile_pair<D>(kb, kb, rowblock_lane_offsets<D>(D * 2, 0, rows_left, src.x, src.y), wave_dst + kRowStage * kStageBytes);
+    issue_tile_pair<D>(vb, vb, rowblock_lane_offsets<D>(vstep, 0, rows_left, src.x, src.y), wave_dst + (kRowStage + 1) * kStageBytes);
   }
   wait_vmcnt<0>();
   __syncthreads();
@@ -496,12 +507,14 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     const int rb = wave & 1;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      kreg[ks] = swz_frag_rm<D>(rm + 2 * kStageBytes, rb, ks);
-      vreg[ks] = swz_frag_rm<D>(rm + 3 * kStageBytes, rb, ks);
+      kreg[ks] = swz_frag_rm<D>(rm + kRowStage * kStageBytes, rb, ks);
+      vreg[ks] = swz_frag_rm<D>(rm + (kRowStage + 1) * kStageBytes, rb, ks);
     }
   }
-  __syncthreads();  // stages 2 and 3 are free again
-  if (n_it > 2) issue_next();
+  __syncthreads();  // the borrowed stages are free again
+#pragma unroll
+  for (int t = R.early_tiles; t < R.startup_tiles; ++t)
+    if (t < n_it) issue_next();
   f32x16 dvacc[MB], dkacc[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) { dvacc[mb] = splat16(0.f); dkacc[mb] = splat16(0.f); }
@@ -599,7 +612,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
       if (MASK == 1 && kw0 > i0 + 31 + p.q_start) request_rowmajor(rm, 1); else step(masked_c, tr, st, 0, i0, rm, 1);
       if (MASK == 1 && kw0 > i0 + 63 + p.q_start) request_rowmajor(rm_lane + nstage * kStageBytes, 0);
       else step(masked_c, tr, st, 1, i0 + 32, rm_lane + nstage * kStageBytes, 0);
-      if (it + 3 < n_it) { issue_next(); wait_vmcnt<kLoadsPerTile>(); } else wait_vmcnt<0>();
+      if (it + R.issue_ahead < n_it) { issue_next(); wait_vmcnt<ring::loads_kept_after_iteration(R, true)>(); } else wait_vmcnt<ring::loads_kept_after_iteration(R, false)>();
       __syncthreads();
       stage = nstage;
     }

@@ -10,6 +10,7 @@
 // Qhat = sm_scale*log2(e) * a_i * q_i * g_q * g_k  (both scale vectors live on the query side) is formed in
 // the prologue; Khat = b_j * k_j and V' = c1 v + c2 v_first are read as written by the pre-pass.
 #include "mfma_common.hpp"
+#include "ring_protocol.hpp"
 
 namespace segpt {
 namespace {
@@ -117,17 +118,18 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
   // same time, the scale vector behind them: one memory round trip.  The remaining start-up tiles follow once the
   // query rows sit in registers (run() below).
   constexpr int kQStages = BQ / 128;            // 128 rows (two tiles) per stage
-  constexpr int kEarlyTiles = NS - (kQStages > 1 ? kQStages : 1);  // of the NS-1 start-up tiles
-  static_assert(kEarlyTiles >= 2 && kEarlyTiles <= NS - kQStages, "start-up tiles and the query block share the ring");
+  constexpr ring::Protocol R = ring::forward(NS, kQStages, Z::kPasses);  // the pipeline's numbers: ring_protocol.hpp
+  static_assert(ring::well_formed(R) && R.loads_per_tile == kLoadsPerTile && !R.wait_before_loop && R.issue_at_top, "tile pipeline");
+  static_assert(R.early_tiles >= ring::kTilesNeededAtLoopStart, "the loop is entered without a further wait");
 #pragma unroll
-  for (int t = 0; t < kEarlyTiles; ++t)
+  for (int t = 0; t < R.early_tiles; ++t)
     if (t < n_kt) issue_tile(t);
   {
     const char* qb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.q, b, h, q0));
 #pragma unroll
     for (int i = 0; i < kQStages; ++i)
       issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, 128 * i, p.Sq - q0, src.x, src.y),
-                         wave_dst + (NS - kQStages + i) * kStageBytes);
+                         wave_dst + (R.row_stage_first + i) * kStageBytes);
   }
 
   // ---- Qhat registers: B operands of S^T, [nb][ks]
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
     const int row = min(qw0 + 32 * nb + ln, p.Sq - 1);
     // rows 32*(NQB*wave + nb) .. +31 of the block: 64-row tile (that / 2), row block (that & 1)
     const int blk = NQB * wave + nb, tile = blk >> 1, rb = blk & 1;
-    const uint32_t rm = lds0 + (NS - kQStages + (tile >> 1)) * kStageBytes + (tile & 1) * Z::kTileBytes + swz_off_rm<D>(lane);
+    const uint32_t rm = lds0 + (R.row_stage_first + (tile >> 1)) * kStageBytes + (tile & 1) * Z::kTileBytes + swz_off_rm<D>(lane);
     u32x4 raw[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) raw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm, rb, ks));
@@ -285,7 +287,7 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
   auto run = [&](auto bounded_c) {
     __syncthreads();  // every wave has its query rows in registers: their stages are free
 #pragma unroll
-    for (int t = kEarlyTiles; t < NS - 1; ++t)
+    for (int t = R.early_tiles; t < R.startup_tiles; ++t)
       if (t < n_kt) issue_tile(t);
     if (n_act > 0) request_rowmajor(rm_lane, 0);
     int stage = 0;
@@ -296,23 +298,23 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
     int jt = 0;
     for (; jt < n_a; ++jt) {
       const int nstage = stage == NS - 1 ? 0 : stage + 1;
-      const bool issued = jt + NS - 1 < n_kt;
-      if (issued) issue_tile(jt + NS - 1);
+      const bool issued = jt + R.issue_ahead < n_kt;
+      if (issued) issue_tile(jt + R.issue_ahead);
       const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
       step(IC<0>{}, bounded_c, tr, 0, 64 * jt, rm, 1);
       step(IC<0>{}, bounded_c, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
-      if (issued) wait_vmcnt<(NS - 3) * kLoadsPerTile>(); else wait_vmcnt<0>();
+      if (issued) wait_vmcnt<ring::loads_kept_after_iteration(R, true)>(); else wait_vmcnt<ring::loads_kept_after_iteration(R, false)>();
       __syncthreads();
       stage = nstage;
     }
     for (; jt < n_kt; ++jt) {
       const int nstage = stage == NS - 1 ? 0 : stage + 1;
-      const bool issued = jt + NS - 1 < n_kt;
-      if (issued) issue_tile(jt + NS - 1);
+      const bool issued = jt + R.issue_ahead < n_kt;
+      if (issued) issue_tile(jt + R.issue_ahead);
       const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
       if (2 * jt < n_act) step(IC<1>{}, bounded_c, tr, 0, 64 * jt, rm, 1);
       if (2 * jt + 1 < n_act) step(IC<1>{}, bounded_c, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
-      if (issued) wait_vmcnt<(NS - 3) * kLoadsPerTile>(); else wait_vmcnt<0>();
+      if (issued) wait_vmcnt<ring::loads_kept_after_iteration(R, true)>(); else wait_vmcnt<ring::loads_kept_after_iteration(R, false)>();
       __syncthreads();
       stage = nstage;
     }
