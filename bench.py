@@ -33,10 +33,73 @@ if ROOT not in sys.path:
 
 MI355X_BF16_DENSE_TFLOPS = 2516.6  # 256 CU x 4096 FLOP/clk/CU x 2.4 GHz (vendor dense figure, no sparsity)
 MI355X_HBM_GBS = 8000.0
-# HBM bytes per launch (read + write) at cfg 3, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a plain
-# copy kernel of known size (FETCH_SIZE reads 0.5 of the true bytes on this part, WRITE_SIZE 1.0); profiler numbers,
-# not measured by this script
-PMC_TRAFFIC_BYTES_CFG3 = {"fwd": 120.1e6, "bwd_dq": 266.3e6, "bwd_dkdv": 208.0e6}
+# HBM bytes per launch (read + write) at cfg 3: profiler numbers, not measured by this script.  The file is written by
+# `bench.py --traffic-from <FETCH_SIZE run> <WRITE_SIZE run>` from two rocprofv3 --pmc runs of this same script (each
+# counter scaled by what it reads for the plain copy of --copy-mib), next to the summary it belongs to.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "imu1_fwd_bwd_hbm_traffic_pmc.json")
+KERNEL_OF_STAGE = {"kv_prep": "kv_prep_kernel", "fwd": "fwd_bf16_kernel", "bwd_dq": "bwd_dq_bf16_kernel", "bwd_dkdv": "bwd_dkdv_bf16_kernel"}
+
+
+def pmc_traffic_bytes(stage):
+    """Measured HBM bytes per launch of the kernel behind `stage` at cfg 3, or None when no profile is on file."""
+    try:
+        d = json.load(open(TRAFFIC_JSON))
+        k = d["kernels"][KERNEL_OF_STAGE[stage]]
+        return round((k["read_mb"] + k["write_mb"]) * 1e6)
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def traffic_from_pmc(fetch_dir, write_dir, copy_mib):
+    """Turns two `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --kernel-trace --output-format csv -d <dir> -- python3 bench.py
+    --copy-mib N ...` runs into HBM bytes per launch: per kernel the mean counter value per dispatch (KiB), scaled by
+    the factor the same counter shows for the plain N-MiB device copy of that run.  Writes TRAFFIC_JSON and prints
+    the table.  Needs no GPU."""
+    import collections
+    import csv
+    import glob
+
+    def per_kernel(d, counter):
+        files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            raise SystemExit(f"no *counter_collection.csv under {d}")
+        acc = collections.defaultdict(list)
+        for r in csv.DictReader(open(files[0])):
+            if r["Counter_Name"] == counter:
+                acc[r["Kernel_Name"]].append(float(r["Counter_Value"]))
+        if not acc:
+            raise SystemExit(f"{files[0]} holds no {counter} rows")
+        return acc
+
+    true_kib = copy_mib * 1024.0
+    out = {"copy_mib": copy_mib, "kernels": {}}
+    vals = {}
+    for counter, d in (("FETCH_SIZE", fetch_dir), ("WRITE_SIZE", write_dir)):
+        acc = per_kernel(d, counter)
+        # the calibration dispatch: the plain copy of copy_mib reads (and writes) exactly that much; it is the largest
+        # dispatch of the runtime's copy kernel (the others are the small input uploads)
+        cal = [max(v) for k, v in acc.items() if "copy" in k.lower()]
+        if not cal or max(cal) <= 0:
+            raise SystemExit(f"no copy kernel found in the {counter} run: was it made with --copy-mib {copy_mib}?")
+        factor = true_kib / max(cal)
+        out[counter + "_factor"] = round(factor, 4)
+        for k, v in acc.items():
+            vals.setdefault(k, {})[counter] = (sum(v) / len(v), len(v))
+        vals["__factor__" + counter] = factor
+    print(f"| kernel | FETCH_SIZE KiB | WRITE_SIZE KiB | read MB (x{out['FETCH_SIZE_factor']}) | write MB (x{out['WRITE_SIZE_factor']}) | launches |")
+    print("|---|---|---|---|---|---|")
+    for short in KERNEL_OF_STAGE.values():
+        match = [k for k in vals if short in k and "FETCH_SIZE" in vals[k] and "WRITE_SIZE" in vals[k]]
+        if not match:
+            continue
+        f, nf = vals[match[0]]["FETCH_SIZE"]
+        w, nw = vals[match[0]]["WRITE_SIZE"]
+        rd = f * 1024 * vals["__factor__FETCH_SIZE"] / 1e6
+        wr = w * 1024 * vals["__factor__WRITE_SIZE"] / 1e6
+        out["kernels"][short] = {"fetch_kib": round(f, 1), "write_kib": round(w, 1), "read_mb": round(rd, 1), "write_mb": round(wr, 1)}
+        print(f"| {short} | {f:.1f} | {w:.1f} | {rd:.1f} | {wr:.1f} | {nf} / {nw} |")
+    json.dump(out, open(TRAFFIC_JSON, "w"), indent=1)
+    print("wrote", os.path.relpath(TRAFFIC_JSON, ROOT))
 
 
 def cpu_baseline(c, batches: int, budget_s: float = 12.0):
@@ -47,6 +110,13 @@ def cpu_baseline(c, batches: int, budget_s: float = 12.0):
     from oracle import qknorm_attn_oracle as orc
     from sample_efficient_gpt_amd import make_inputs
 
+    # every host core this process may use: os.cpu_count(), cut down to the scheduler affinity and to the thread budget
+    # the box exports (OMP_NUM_THREADS: a 1-GPU box shares its host, and oversubscribing the share only slows the run)
+    host_cores = os.cpu_count() or 1
+    usable = min(host_cores, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else host_cores)
+    if os.environ.get("OMP_NUM_THREADS", "").isdigit():
+        usable = max(1, min(usable, int(os.environ["OMP_NUM_THREADS"])))
+    torch.set_num_threads(usable)
     cs = c.scaled(B=batches)
     x = make_inputs(cs)
     f = lambda n: x[n].float()
@@ -68,11 +138,41 @@ def cpu_baseline(c, batches: int, budget_s: float = 12.0):
         "value": round(passes * cs.flops() / dt / 1e12, 5),
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
+        "host_cores": host_cores,
+        "parallel_info": torch.__config__.parallel_info().strip().splitlines()[0],
         "kind": "port",
         "sample": f"{passes} passes over {batches} of {c.B} batches of the same workload, fp32, fwd{'+bwd' if c.backward else ''} "
                   f"({dt:.1f} s in all): RMS-normalise + F.scaled_dot_product_attention(is_causal) + autograd",
         "seconds": round(dt, 3),
     }
+
+
+def module_shaped_inputs(c, dev):
+    """Operands laid out as MultiHeadSelfAttention hands them to the kernels (module.py, following the reference's
+    attention.py:186-255): q / k / v are strided [B, heads, S, D] views of ONE projection output [B, S, (H+2Hkv) D];
+    v_first is the v slice of another layer's projection; d_o arrives in [B, S, H, D] layout (the gradient of the
+    `b seq (h d)` tensor the output projection consumed); gain is the module's scalar.  Returns (x, (cos, sin))."""
+    import torch
+
+    g = torch.Generator().manual_seed(2000 + c.cfg)
+    n = lambda *s: torch.randn(*s, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    B, S, H, Hkv, D = c.B, c.S, c.H, c.Hkv, c.D
+
+    def split(proj):
+        q = proj[..., : H * D].unflatten(-1, (H, D)).permute(0, 2, 1, 3)
+        k = proj[..., H * D : (H + Hkv) * D].unflatten(-1, (Hkv, D)).permute(0, 2, 1, 3)
+        v = proj[..., (H + Hkv) * D :].unflatten(-1, (Hkv, D)).permute(0, 2, 1, 3)
+        return q, k, v
+
+    q, k, v = split(n(B, S, (H + 2 * Hkv) * D))
+    _, _, v_first = split(n(B, S, (H + 2 * Hkv) * D))
+    lam = 0.3 + 0.4 * torch.rand(1, generator=g)
+    x = {"q": q, "k": k, "v": v, "v_first": v_first, "g_q": torch.ones(1) + 0.02 * torch.randn(1, generator=g),
+         "gate_logits": n(B, S, H), "vr_coef": torch.cat([lam, 1.0 - lam]).to(dev),
+         "d_o": n(B, S, H, D).permute(0, 2, 1, 3)}
+    j = torch.arange(0, D // 2)
+    ang = torch.outer(torch.arange(S), 10_000.0 ** (-2 * j / D))  # rope.py:12-34
+    return x, (ang.cos().float().to(dev), ang.sin().float().to(dev))
 
 
 def _read_sclk_mhz():
@@ -170,6 +270,15 @@ def main():
                     help="instead of a training config: one generation step (1 new token per sequence, IMU-1 heads) "
                          "against a cache of this many keys, through the split-key decode kernels; reports K+V GB/s")
     ap.add_argument("--decode-batch", type=int, default=8)
+    ap.add_argument("--module-shaped", action="store_true",
+                    help="the call MultiHeadSelfAttention makes (reference: attention.py:186-204,243-255 with the IMU-1 "
+                         "model's switches, configs/imu1_base.yaml:9-11): q / k / v as strided views of one "
+                         "[B, S, (H + 2 Hkv) D] projection buffer, rotary embedding applied in the loads, scalar gain, "
+                         "per-head gate, value residual against another layer's strided v, output and dY in "
+                         "[B, S, H D] layout; same shape and credited FLOPs as the chosen config")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="no benchmark: summarise two rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE; both "
+                         "made with --copy-mib N, pass the same N here) into profiles/imu1_fwd_bwd_hbm_traffic_pmc.json")
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known traffic, for scaling "
                          "the profiler's FETCH_SIZE / WRITE_SIZE counters)")
@@ -178,6 +287,11 @@ def main():
         print("bench.py: this build runs on ONE GPU only (the attention path has no cross-GPU step); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.traffic_from:
+        if args.copy_mib <= 0:
+            raise SystemExit("--traffic-from needs the --copy-mib value the two profiler runs were made with")
+        return traffic_from_pmc(args.traffic_from[0], args.traffic_from[1], args.copy_mib)
 
     import torch
 
@@ -192,12 +306,19 @@ def main():
     if args.batch > 0:
         c = c.scaled(B=args.batch)
     resized = args.seq_len > 0 or args.batch > 0
+    if args.module_shaped:
+        c = c.scaled(extras=True)  # gate + value residual, as the IMU-1 model has them
     if c.dtype != torch.bfloat16 and args.cfg != 1:
         raise SystemExit("unsupported config")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    x = make_inputs(c, device=dev)
-    plan = AttnPlan(x, eps=c.eps, sm_scale=c.sm_scale, gate_scale=c.gate_scale, backward=c.backward)
+    if args.module_shaped:
+        x, rope = module_shaped_inputs(c, dev)
+        plan = AttnPlan(x, eps=c.eps, sm_scale=c.sm_scale, gate_scale=2.0, backward=c.backward,
+                        rope_cos=rope[0], rope_sin=rope[1], rope_q_pos0=0, rope_k_pos0=0)
+    else:
+        x = make_inputs(c, device=dev)
+        plan = AttnPlan(x, eps=c.eps, sm_scale=c.sm_scale, gate_scale=c.gate_scale, backward=c.backward)
     names = ["kv_prep", "fwd"] + (["bwd_dq", "bwd_dkdv", "bwd_reduce"] if c.backward else [])
 
     def step_plain():  # the product's two entry points; the backward reuses the forward's normalised keys
@@ -225,6 +346,18 @@ def main():
         del src, dst
     # untimed pre-warm: a fresh box idles at ~1.46 GHz and takes a few milliseconds of load to reach its working
     # clock; W = 5 warm-up steps are 2 ms.  Not part of `warmup` or of the timed region.
+    # The same W + K steps as below, but from the idle clock (what a run without the pre-warm reports): kept beside the
+    # headline so that the pre-warm reads as what it is, a change of the measurement and not of the kernels.
+    ms_cold = None
+    if args.prewarm > 0:
+        for _ in range(args.warmup):
+            step_plain()
+        torch.cuda.synchronize()
+        tc = time.perf_counter()
+        for _ in range(args.steps):
+            step_plain()
+        torch.cuda.synchronize()
+        ms_cold = (time.perf_counter() - tc) / args.steps * 1e3
     prewarm_steps = 0
     tw = time.perf_counter()
     while time.perf_counter() - tw < args.prewarm:
@@ -316,7 +449,8 @@ def main():
 
     out = {
         "metric": "attention fwd+bwd TFLOP/s at IMU-1 shape, 1 GPU" if args.cfg == 3 and not resized
-                  else f"attention TFLOP/s, cfg {args.cfg}" + (" resized" if resized else ""),
+                  and not args.module_shaped
+                  else f"attention TFLOP/s, cfg {args.cfg}" + (" resized" if resized else "") + (" module-shaped" if args.module_shaped else ""),
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -331,12 +465,15 @@ def main():
         "config": {
             "workload": f"cfg{c.cfg} {c.name}: B={c.B} S={c.S} q_heads={c.H} kv_heads={c.Hkv} head_dim={c.D} causal "
                         f"QK-norm (vector scales, eps 1e-6){' + per-head gate + value residual' if c.extras else ''}, "
-                        f"{'forward + backward' if c.backward else 'forward only'}",
+                        f"{'forward + backward' if c.backward else 'forward only'}"
+                        + ("; MODULE-SHAPED call: strided q/k/v views of one projection buffer, rotary embedding in the "
+                           "loads, scalar gain, per-head gate, value residual, [B,S,H*D] output layout" if args.module_shaped else ""),
             "algorithmic_flops_per_step": total_flops,
         },
         "pct_of_bf16_mfma_peak": round(100 * value / MI355X_BF16_DENSE_TFLOPS, 2),
         "prewarm_s": args.prewarm,
         "prewarm_steps": prewarm_steps,
+        "ms_per_step_from_idle_clock": None if ms_cold is None else round(ms_cold, 5),
         "sclk_mhz_under_load": sclk,
         "launch_mode": launch_mode,
         "ms_per_step_eager": round(ms_eager, 5),
@@ -352,7 +489,7 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(achieved / MI355X_BF16_DENSE_TFLOPS, 4),
             "sclk_mhz_under_load": sclk,  # the peak assumes 2400 MHz
-            "traffic": PMC_TRAFFIC_BYTES_CFG3.get(dom) if args.cfg == 3 and not resized else None,
+            "traffic": pmc_traffic_bytes(dom) if args.cfg == 3 and not resized and not args.module_shaped else None,
             "credited_flops_per_launch": credited[dom],
             "avg_launch_ms": round(kern_ms[dom], 5),
             "timing": "HIP events between the stages, second pass over the same K steps, minus the cost of an empty event pair",
