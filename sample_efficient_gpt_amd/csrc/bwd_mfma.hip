@@ -45,7 +45,10 @@ constexpr int kStages = 4;  // LDS ring of streamed stages (two tiles each): til
 //   A(n+1) request the row-major fragments of block n+1 (possibly the next tile, already in LDS)
 //   E(n)  T^T += Khat^T dS^T MFMAs
 // Tiles travel global->LDS directly (no registers), three tiles ahead of their use.
-template <int D>
+// ROPE (rope tables given) is a compile-time switch so that the table rows are ordinary, unconditional loads which
+// travel with the start-up tiles (prologue) and with the first stores (epilogue) instead of costing a memory round
+// trip of their own behind a branch.
+template <int D, bool ROPE>
 __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel(KArgs a) {
   using Z = Swz<D>;
   constexpr int BQ = kBwdRows;
@@ -127,6 +130,9 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     issue_tile_pair<D>(yb, yb, rowblock_lane_offsets<D>((uint32_t)p.o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + (kRowStage + 2) * kStageBytes);
   }
   const float lse_row = p.lse[ridx];
+  const int64_t rope_pos = ROPE ? (int64_t)(p.rope_q_pos0 + row_c) * (D / 2) : 0;
+  RopeB<KS> rope_b;
+  if (ROPE) rope_b = rope_b_load<KS>(p.rope_cos + rope_pos, p.rope_sin + rope_pos, hh);
   // the conditional reads last: the compiler waits for every outstanding load where their branches join
   float gate_z = 0.f;
   if (p.gate.ptr)
@@ -170,10 +176,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
       for (int i = 0; i < 4; ++i) dl += bf16lo(yraw[ks][i]) * bf16lo(dyraw[ks][i]) + bf16hi(yraw[ks][i]) * bf16hi(dyraw[ks][i]);
     float qx[KS][8];
     unpack_b_layout<KS>(qraw, qx);
-    if (p.rope_cos) {
-      const int64_t pos = (int64_t)(p.rope_q_pos0 + row_c) * (D / 2);
-      rope_b_layout<KS>(qx, p.rope_cos + pos, p.rope_sin + pos, hh);
-    }
+    if (ROPE) rope_b_apply<KS>(qx, rope_b);
     float ss = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
@@ -298,6 +301,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   }
 
   // ---- epilogue.  First what the dK/dV kernel reads of this row: Qhat, the gated dO, -delta, -lse2 (and dgate).
+  RopeCt<MB> rope_ct;
+  if (ROPE) rope_ct = rope_ct_load<MB>(p.rope_cos + rope_pos, p.rope_sin + rope_pos, hh);
   if (live) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -320,14 +325,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) unpack_ct_block(qct[mb], qv[mb]);
   const float aq = live ? alpha : 0.f;  // padding rows add nothing to the scale gradient
-  const float* cosr = nullptr;
-  const float* sinr = nullptr;
-  if (p.rope_cos) {
-    const int64_t pos = (int64_t)(p.rope_q_pos0 + row_c) * (D / 2);
-    cosr = p.rope_cos + pos;
-    sinr = p.rope_sin + pos;
-    rope_ct_layout<MB, false>(qv, cosr, sinr, hh);
-  }
+  if (ROPE) rope_ct_apply<MB, false>(qv, rope_ct);
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
@@ -355,7 +353,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) val[mb][r] = alpha * acc[mb][r] - a3 * qv[mb][r];
-  if (p.rope_cos) rope_ct_layout<MB, true>(val, cosr, sinr, hh);
+  if (ROPE) rope_ct_apply<MB, true>(val, rope_ct);
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) store_ct_block(op, mb, hh, live, val[mb]);
   // workgroup partial of dg: column sums over the 128 (wave, lane%32) rows, in two levels so that all
@@ -384,7 +382,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
 // Same pipeline with the roles swapped: the streamed tiles are Qhat / dO (64 queries of one head), the
 // blocks are 32 queries, and B(n) starts from the two row statistics of the block, read from LDS
 // straight into the accumulators of S and dP.
-template <int D>
+template <int D, bool ROPE>
 __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kernel(KArgs a) {
   using Z = Swz<D>;
   constexpr int BKV = kBwdRows;
@@ -667,13 +665,11 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     float kv[MB][16];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) load_ct_block(kp, mb, hh, kv[mb]);
-    const float* cosr = nullptr;
-    const float* sinr = nullptr;
-    if (p.rope_cos) {  // the normaliser acted on the rotated key: work in that frame, rotate the gradient back
+    RopeCt<MB> rope_ct;
+    if (ROPE) {  // the normaliser acted on the rotated key: work in that frame, rotate the gradient back
       const int64_t pos = (int64_t)(p.rope_k_pos0 + key_c) * (D / 2);
-      cosr = p.rope_cos + pos;
-      sinr = p.rope_sin + pos;
-      rope_ct_layout<MB, false>(kv, cosr, sinr, hh);
+      rope_ct = rope_ct_load<MB>(p.rope_cos + pos, p.rope_sin + pos, hh);
+      rope_ct_apply<MB, false>(kv, rope_ct);
     }
     float dot = 0.f, ss = 0.f;
 #pragma unroll
@@ -690,7 +686,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) val[mb][r] = beta * kLn2 * dkacc[mb][r] - b3 * kv[mb][r];
-    if (p.rope_cos) rope_ct_layout<MB, true>(val, cosr, sinr, hh);
+    if (ROPE) rope_ct_apply<MB, true>(val, rope_ct);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) store_ct_block(okp, mb, hh, live, val[mb]);
   }
@@ -700,7 +696,9 @@ template <int D>
 int launch_dkdv_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
   const int n_kvt = (p.Sk + kBwdRows - 1) / kBwdRows;
-  hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D>), dim3((unsigned)(wg_grid(n_kvt, p.B, p.Hkv, 1, dkdv_pinned(p)) + 1)), dim3(kThreadsM), 0, st, a);
+  const dim3 grid((unsigned)(wg_grid(n_kvt, p.B, p.Hkv, 1, dkdv_pinned(p)) + 1));
+  if (p.rope_cos) hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D, true>), grid, dim3(kThreadsM), 0, st, a);
+  else hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<D, false>), grid, dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 
@@ -708,7 +706,9 @@ template <int D>
 int launch_dq_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
   const int n_qt = (p.Sq + kBwdRows - 1) / kBwdRows;
-  hipLaunchKernelGGL((bwd_dq_bf16_kernel<D>), dim3((unsigned)wg_grid(n_qt, p.B, p.Hkv, p.H / p.Hkv, wg_pinned_pairs(p.B, p.Hkv, false))), dim3(kThreadsM), 0, st, a);
+  const dim3 grid((unsigned)wg_grid(n_qt, p.B, p.Hkv, p.H / p.Hkv, wg_pinned_pairs(p.B, p.Hkv, false)));
+  if (p.rope_cos) hipLaunchKernelGGL((bwd_dq_bf16_kernel<D, true>), grid, dim3(kThreadsM), 0, st, a);
+  else hipLaunchKernelGGL((bwd_dq_bf16_kernel<D, false>), grid, dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 

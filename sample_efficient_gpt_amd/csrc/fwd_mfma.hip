@@ -66,7 +66,9 @@ struct FwdShape {
   static constexpr int kBQ = 4 * 32 * kNQB;
 };
 
-template <int D, bool WIDE>
+// ROPE (rope tables given) is a compile-time switch so that the table rows are ordinary, unconditional loads that
+// travel with the start-up tiles instead of costing a memory round trip of their own behind a branch.
+template <int D, bool WIDE, bool ROPE>
 __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16_kernel(KArgs a) {
   using Z = Swz<D>;
   using F = FwdShape<D, WIDE>;
@@ -133,6 +135,14 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
   }
 
   // ---- Qhat registers: B operands of S^T, [nb][ks]
+  RopeB<KS> rope_b[NQB];
+  if (ROPE) {
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+      const int64_t pos = (int64_t)(p.rope_q_pos0 + min(qw0 + 32 * nb + ln, p.Sq - 1)) * (D / 2);
+      rope_b[nb] = rope_b_load<KS>(p.rope_cos + pos, p.rope_sin + pos, hh);
+    }
+  }
   float gval = 0.f;
   if (tid < D) gval = gprod_at(p, tid) * p.sm_scale * kLog2e;
   if (tid < D) gsm[tid] = gval;
@@ -151,10 +161,7 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
     for (int ks = 0; ks < KS; ++ks) raw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm, rb, ks));
     float x[KS][8];
     unpack_b_layout<KS>(raw, x);
-    if (p.rope_cos) {
-      const int64_t pos = (int64_t)(p.rope_q_pos0 + row) * (D / 2);
-      rope_b_layout<KS>(x, p.rope_cos + pos, p.rope_sin + pos, hh);
-    }
+    if (ROPE) rope_b_apply<KS>(x, rope_b[nb]);
     float ss = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
@@ -349,7 +356,9 @@ template <int D, bool WIDE>
 int launch_fwd_t(const KArgs& a, hipStream_t st) {
   const segpt_attn_params& p = a.p;
   const int n_qt = (p.Sq + FwdShape<D, WIDE>::kBQ - 1) / FwdShape<D, WIDE>::kBQ;
-  hipLaunchKernelGGL((fwd_bf16_kernel<D, WIDE>), dim3((unsigned)wg_grid(n_qt, p.B, p.Hkv, p.H / p.Hkv, wg_pinned_pairs(p.B, p.Hkv, false))), dim3(kThreadsM), 0, st, a);
+  const dim3 grid((unsigned)wg_grid(n_qt, p.B, p.Hkv, p.H / p.Hkv, wg_pinned_pairs(p.B, p.Hkv, false)));
+  if (p.rope_cos) hipLaunchKernelGGL((fwd_bf16_kernel<D, WIDE, true>), grid, dim3(kThreadsM), 0, st, a);
+  else hipLaunchKernelGGL((fwd_bf16_kernel<D, WIDE, false>), grid, dim3(kThreadsM), 0, st, a);
   return (int)hipGetLastError();
 }
 

@@ -213,39 +213,69 @@ __device__ __forceinline__ bf16x8 pack_c_half_sum(const f32x16& c, int s, float 
   return as_bf16x8(w);
 }
 
-// ---- rotary embedding in the two register layouts of a tensor row (cosr / sinr: the table row of the
-// row's position, D/2 floats; both NULL-free: callers test p.rope_cos first)
+// ---- rotary embedding in the two register layouts of a tensor row.  The table entries of the row's position
+// (cosr / sinr: D/2 floats each) are LOADED into registers by one function and APPLIED by another, so that a kernel
+// can request them together with its other start-up loads (one memory round trip) and use them later.
 // B-operand layout: x[ks][t] = element 16 ks + 8 hh + t; the partner of ks is ks + KS/2 in the same lane
 template <int KS>
-__device__ __forceinline__ void rope_b_layout(float (&x)[KS][8], const float* cosr, const float* sinr, int hh) {
+struct RopeB {
+  float c[KS / 2][8], s[KS / 2][8];
+};
+template <int KS>
+__device__ __forceinline__ RopeB<KS> rope_b_load(const float* cosr, const float* sinr, int hh) {
+  RopeB<KS> r;
 #pragma unroll
   for (int ks = 0; ks < KS / 2; ++ks) {
     const float4 c0 = *reinterpret_cast<const float4*>(cosr + 16 * ks + 8 * hh);
     const float4 c1 = *reinterpret_cast<const float4*>(cosr + 16 * ks + 8 * hh + 4);
     const float4 s0 = *reinterpret_cast<const float4*>(sinr + 16 * ks + 8 * hh);
     const float4 s1 = *reinterpret_cast<const float4*>(sinr + 16 * ks + 8 * hh + 4);
-    const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-    const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-#pragma unroll
-    for (int t = 0; t < 8; ++t) rope_pair(x[ks][t], x[ks + KS / 2][t], c[t], sn[t]);
+    r.c[ks][0] = c0.x; r.c[ks][1] = c0.y; r.c[ks][2] = c0.z; r.c[ks][3] = c0.w;
+    r.c[ks][4] = c1.x; r.c[ks][5] = c1.y; r.c[ks][6] = c1.z; r.c[ks][7] = c1.w;
+    r.s[ks][0] = s0.x; r.s[ks][1] = s0.y; r.s[ks][2] = s0.z; r.s[ks][3] = s0.w;
+    r.s[ks][4] = s1.x; r.s[ks][5] = s1.y; r.s[ks][6] = s1.z; r.s[ks][7] = s1.w;
   }
+  return r;
+}
+template <int KS>
+__device__ __forceinline__ void rope_b_apply(float (&x)[KS][8], const RopeB<KS>& r) {
+#pragma unroll
+  for (int ks = 0; ks < KS / 2; ++ks)
+#pragma unroll
+    for (int t = 0; t < 8; ++t) rope_pair(x[ks][t], x[ks + KS / 2][t], r.c[ks][t], r.s[ks][t]);
+}
+template <int KS>
+__device__ __forceinline__ void rope_b_layout(float (&x)[KS][8], const float* cosr, const float* sinr, int hh) {
+  rope_b_apply<KS>(x, rope_b_load<KS>(cosr, sinr, hh));
 }
 // C-tile layout of load_ct_block / store_ct_block: x[mb][4c + i] = element 32 mb + 8 c + 4 hh + i; the
 // partner of mb is mb + MB/2 in the same lane and register
-template <int MB, bool INVERSE>
-__device__ __forceinline__ void rope_ct_layout(float (&x)[MB][16], const float* cosr, const float* sinr, int hh) {
+template <int MB>
+struct RopeCt {
+  float c[MB / 2][16], s[MB / 2][16];
+};
+template <int MB>
+__device__ __forceinline__ RopeCt<MB> rope_ct_load(const float* cosr, const float* sinr, int hh) {
+  RopeCt<MB> r;
 #pragma unroll
   for (int mb = 0; mb < MB / 2; ++mb)
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const float4 c4 = *reinterpret_cast<const float4*>(cosr + 32 * mb + 8 * c + 4 * hh);
       const float4 s4 = *reinterpret_cast<const float4*>(sinr + 32 * mb + 8 * c + 4 * hh);
-      const float cc[4] = {c4.x, c4.y, c4.z, c4.w}, ss[4] = {s4.x, s4.y, s4.z, s4.w};
+      r.c[mb][4 * c] = c4.x; r.c[mb][4 * c + 1] = c4.y; r.c[mb][4 * c + 2] = c4.z; r.c[mb][4 * c + 3] = c4.w;
+      r.s[mb][4 * c] = s4.x; r.s[mb][4 * c + 1] = s4.y; r.s[mb][4 * c + 2] = s4.z; r.s[mb][4 * c + 3] = s4.w;
+    }
+  return r;
+}
+template <int MB, bool INVERSE>
+__device__ __forceinline__ void rope_ct_apply(float (&x)[MB][16], const RopeCt<MB>& r) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (INVERSE) rope_pair_inv(x[mb][4 * c + i], x[mb + MB / 2][4 * c + i], cc[i], ss[i]);
-        else rope_pair(x[mb][4 * c + i], x[mb + MB / 2][4 * c + i], cc[i], ss[i]);
-      }
+  for (int mb = 0; mb < MB / 2; ++mb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if (INVERSE) rope_pair_inv(x[mb][i], x[mb + MB / 2][i], r.c[mb][i], r.s[mb][i]);
+      else rope_pair(x[mb][i], x[mb + MB / 2][i], r.c[mb][i], r.s[mb][i]);
     }
 }
 // raw bf16 words of a B-operand row -> floats

@@ -73,15 +73,21 @@ __global__ __launch_bounds__(256) void kv_prep_kernel(KArgs a) {
   float k[8];
   Elem<uint16_t>::load(row_ptr<uint16_t>(p.k, b, g, s) + part * 8, k);
   if (p.rope_cos) {
-    // split-half pairs (j, j + D/2): the partner element sits TPR/2 lanes away, same slot
+    // split-half pairs (j, j + D/2): the partner element sits TPR/2 lanes away, same slot.  The lane's eight table
+    // entries come in as four 16-byte loads (table rows are 16-byte aligned and jp is a multiple of 8 floats) and the
+    // two halves share one expression, x' = x c + sign * partner * s, so that no lane-dependent branch splits the loads.
     const int jp = (part % (TPR / 2)) * 8;
     const float* cr = p.rope_cos + (int64_t)(p.rope_k_pos0 + s) * (D / 2) + jp;
     const float* sr = p.rope_sin + (int64_t)(p.rope_k_pos0 + s) * (D / 2) + jp;
-    const bool first = part < TPR / 2;
+    const float4 c0 = *reinterpret_cast<const float4*>(cr), c1 = *reinterpret_cast<const float4*>(cr + 4);
+    const float4 s0 = *reinterpret_cast<const float4*>(sr), s1 = *reinterpret_cast<const float4*>(sr + 4);
+    const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+    const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+    const float sign = part < TPR / 2 ? -1.f : 1.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float other = __shfl_xor(k[e], TPR / 2, 64);
-      k[e] = first ? k[e] * cr[e] - other * sr[e] : other * sr[e] + k[e] * cr[e];
+      k[e] = k[e] * cv[e] + sign * other * sv[e];
     }
   }
   float ss = 0.f;
