@@ -90,6 +90,8 @@ int check_t4(const segpt_tensor4& t, const segpt_attn_params& p) {
   const int64_t per16 = 16 / (int64_t)elem_bytes(p);
   if (t.stride_b < 0 || t.stride_h < 0 || t.stride_s < p.D) return SEGPT_E_STRIDE;
   if (t.stride_b % per16 || t.stride_h % per16 || t.stride_s % per16) return SEGPT_E_STRIDE;
+  // the bf16 kernels address the rows of a tile (up to 256 of them) by 32-bit byte offsets from the tile's first row
+  if (p.dtype == SEGPT_DTYPE_BF16 && t.stride_s > (int64_t)(UINT32_MAX / (256 * 2))) return SEGPT_E_STRIDE;
   return SEGPT_OK;
 }
 
@@ -200,7 +202,7 @@ const char* segpt_strerror(int code) {
     case SEGPT_E_DTYPE: return "unknown dtype (expected SEGPT_DTYPE_BF16 or SEGPT_DTYPE_FP32)";
     case SEGPT_E_SHAPE: return "bad shape: sizes must be positive, H divisible by Hkv, scale vectors of 1 or D elements";
     case SEGPT_E_HEAD_DIM: return "unsupported head_dim: bf16 needs D in {64,128}, fp32 D in {32,64,128}";
-    case SEGPT_E_STRIDE: return "bad stride: strides must be non-negative multiples of 16 bytes and rows must not overlap";
+    case SEGPT_E_STRIDE: return "bad stride: strides must be non-negative multiples of 16 bytes, rows must not overlap, and a bf16 row stride must stay below 2^23 elements";
     case SEGPT_E_WORKSPACE: return "workspace or kv_workspace missing or smaller than segpt_attn_workspace_bytes()";
     case SEGPT_E_EXTRAS: return "inconsistent optional operands (v_first/vr_coef/gate and their gradient slots)";
     case SEGPT_E_QSTART: return "q_start must be >= 0";

@@ -91,6 +91,9 @@ def test_argument_errors_are_reported_before_any_launch(lib):
     assert lib.segpt_attn_fwd(p, None) == -6
     p = _valid_params(); p.k.stride_h = 7
     assert lib.segpt_attn_fwd(p, None) == -6
+    # a bf16 row stride whose 256-row tile offsets would not fit 32 bits (the tile loads address rows that way)
+    p = _valid_params(); p.q.stride_s = 1 << 23
+    assert lib.segpt_attn_fwd(p, None) == -6
     # an OUTPUT view must not alias itself (a broadcast or overlapping view would make workgroups race)
     p = _valid_params(); p.o.stride_h = 0
     assert lib.segpt_attn_fwd(p, None) == -6
