@@ -214,7 +214,12 @@ int segpt_attn_fwd_stage(const segpt_attn_params* p, int stage, void* stream);
  * a shape whose segpt_attn_workspace_bytes(p, SEGPT_WS_KV) exceeds the array returns SEGPT_E_SCRATCH_LIMIT
  * before any launch.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (different
  * streams or threads) race, and no later call may rely on its contents (SEGPT_FLAG_KV_PREPARED is ignored here, and
- * a backward must run its own key/value pre-pass on a caller-owned kv_workspace). */
+ * a backward must run its own key/value pre-pass on a caller-owned kv_workspace).
+ * The array that is used is the CURRENT device's (hipGetDevice), so `stream` must be a stream of the current device
+ * (another device's stream returns hipErrorInvalidDevice).  The first call on each device looks the array's address
+ * up (hipGetSymbolAddress) and keeps it: make that first call outside stream capture; later calls are plain kernel
+ * launches and may be captured into a HIP graph and replayed.  The array is part of the library's device image and
+ * occupies its SEGPT_NOALLOC_SCRATCH_BYTES on every GPU the library is loaded on, used or not. */
 int segpt_attn_fwd_noalloc(const segpt_attn_params* p, void* stream);
 
 #ifdef __cplusplus

@@ -250,8 +250,10 @@ int segpt_attn_fwd(const segpt_attn_params* p, void* stream) {
   return fwd_stage_impl(p, SEGPT_FWD_STAGE_PRE, SEGPT_FWD_STAGE_ATTN, stream);
 }
 
-// Device address of `scratch` on the current device, looked up once per device (first call there).
-static int noalloc_scratch_ptr(void** out) {
+// Device address of `scratch` on the CURRENT device, looked up once per device (first call there).  Kernels are
+// launched on `stream`, so the stream has to belong to the current device: a stream of another GPU would run them
+// against this GPU's copy of the array, and is refused.
+static int noalloc_scratch_ptr(void** out, hipStream_t stream) {
   constexpr int kMaxDevices = 64;
   static std::mutex mu;
   static void* ptrs[kMaxDevices] = {};
@@ -259,6 +261,10 @@ static int noalloc_scratch_ptr(void** out) {
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return (int)e;
   if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+  if (stream) {  // the null stream is the current device's by definition
+    hipDevice_t sdev = -1;
+    if (hipStreamGetDevice(stream, &sdev) == hipSuccess && (int)sdev != dev) return (int)hipErrorInvalidDevice;
+  }
   std::lock_guard<std::mutex> lock(mu);
   if (!ptrs[dev]) {
     void* ptr = nullptr;
@@ -287,7 +293,7 @@ int segpt_attn_fwd_noalloc(const segpt_attn_params* p, void* stream) {
     if (!rc) rc = check_t4_out(q.o, q, q.H, q.Sq);
     if (rc) return rc;
     void* ptr = nullptr;
-    if ((rc = noalloc_scratch_ptr(&ptr))) return rc;
+    if ((rc = noalloc_scratch_ptr(&ptr, reinterpret_cast<hipStream_t>(stream)))) return rc;
     q.kv_workspace = ptr;
   }
   return fwd_stage_impl(&q, SEGPT_FWD_STAGE_PRE, SEGPT_FWD_STAGE_ATTN, stream);

@@ -166,12 +166,14 @@ class _GradModeAtApply:
     _tls = threading.local()
 
     @classmethod
+    @torch.compiler.disable  # Python-side bookkeeping the compiler cannot trace: a compiled caller breaks the graph here
     def apply(cls, *args, **kwargs):
+        outer = getattr(cls._tls, "inference", False)  # a nested apply must leave the outer call's decision in place
         cls._tls.inference = _no_backward_will_follow(*(a for a in args if isinstance(a, torch.Tensor)))
         try:
             return super().apply(*args, **kwargs)
         finally:
-            cls._tls.inference = False
+            cls._tls.inference = outer
 
     @classmethod
     def _inference(cls):

@@ -65,13 +65,20 @@ class KVCache:
         self.keys, self.values = self._kbuf[:, :, :need], self._vbuf[:, :, :need]
         return self.keys, self.values
 
+    @property
+    def mixed_length(self):
+        """Rows of the mixed value tensor kept so far (see ``append_mixed``)."""
+        return self._mlen
+
     def append_mixed(self, vm_new):
-        """Rows [length - S, length) of the mixed value tensor (the ``V`` a value-residual layer returns for later
+        """Rows [mixed_length, length) of the mixed value tensor (the ``V`` a value-residual layer returns for later
         layers, attention.py:228,267), kept beside the raw values so that a generation step mixes only its new
-        rows instead of the whole cache.  Call after ``append`` of the same step; returns the ``[B, Hkv, length, D]``
-        view."""
+        rows instead of the whole cache.  Call after ``append`` of the same step with exactly the rows that are
+        missing (``length - mixed_length`` of them: more than the step's own when earlier steps did not keep
+        theirs, e.g. a prefill that ran with gradients enabled); returns the ``[B, Hkv, length, D]`` view."""
         S = vm_new.shape[2]
-        assert self._mlen + S == self.length, "append_mixed follows append, once per step"
+        if self._mlen + S != self.length:
+            raise ValueError(f"append_mixed got {S} rows, the cache is missing rows [{self._mlen}, {self.length})")
         if self._mbuf is None or self._mbuf.shape[2] < self._vbuf.shape[2]:
             mb = torch.empty_like(self._vbuf)
             if self._mbuf is not None:
@@ -200,7 +207,10 @@ class MultiHeadSelfAttention(nn.Module):
             if v_mixed is not None:
                 mix = lambda a, f: (vr_coef[0] * a.float() + vr_coef[1] * f.float()).to(v.dtype)
                 if kv_cache is not None and v1 is None and not torch.is_grad_enabled():
-                    v_mixed = kv_cache.append_mixed(mix(v[:, :, q_start:], v_first[:, :, q_start:]))
+                    # every row the cache does not hold yet: the step's own, and any that earlier steps mixed
+                    # outside the cache (a prefill with gradients enabled takes the full mix below)
+                    m0 = kv_cache.mixed_length
+                    v_mixed = kv_cache.append_mixed(mix(v[:, :, m0:], v_first[:, :, m0:]))
                 else:
                     v_mixed = mix(v, v_first)
         gate_logits = None

@@ -388,6 +388,46 @@ def test_library_op_compiled_and_checkpointed_matches_eager(gpu_device):
         assert torch.equal(a, b)
 
 
+def test_positional_dropin_functions_under_torch_compile(gpu_device):
+    """The positional drop-ins (`QKNormFlashAttnFunc.apply`, `FlashAttnFunc.apply`) called from a compiled function:
+    their `apply` records the caller's grad mode in Python, which the compiler may only run by breaking the graph
+    around the call (no fullgraph here); outputs and gradients must equal the eager call bit for bit, for a call
+    that is followed by a backward and for one under no_grad."""
+    H, B, S, d = 4, 2, 136, 64
+    g = torch.Generator().manual_seed(33)
+    mk = lambda: torch.randn(H * B, S, d, generator=g).to(BF16).to(gpu_device)
+    Q, K, V, dO = mk(), mk(), mk(), mk()
+    gain = torch.full((1,), 1.1, device=gpu_device)
+
+    def f_norm(q, k, v, gn):
+        return QKNormFlashAttnFunc.apply(q * 1, k, v, gn, True, 0)
+
+    def f_plain(q, k, v):
+        return FlashAttnFunc.apply(q * 1, k, v, 0, True)
+
+    def run(fn, *args):
+        leaves = [a.detach().clone().requires_grad_(True) for a in args]
+        y = fn(*leaves)
+        y.backward(dO)
+        return [y.detach()] + [l.grad for l in leaves]
+
+    for fn, args in ((f_norm, (Q, K, V, gain)), (f_plain, (Q, K, V))):
+        ref = run(fn, *args)
+        got = run(torch.compile(fn, backend="aot_eager"), *args)
+        for a, b in zip(ref, got):
+            assert torch.equal(a, b)
+        with torch.no_grad():
+            assert torch.equal(fn(*args), torch.compile(fn, backend="aot_eager")(*args))
+    # a nested apply leaves the outer call's decision in place
+    QKNormFlashAttnFunc._tls.inference = True
+    try:
+        with torch.no_grad():
+            FlashAttnFunc.apply(Q, K, V, 0, True)
+        assert QKNormFlashAttnFunc._inference() is True
+    finally:
+        QKNormFlashAttnFunc._tls.inference = False
+
+
 # ------------------------------------------------------------------ rotary embedding fused into the loads
 
 
@@ -926,6 +966,30 @@ def test_mhsa_module_generation_with_cache(gpu_device):
     wd = {n: t.detach() for n, t in w.items()}
     ref, _ = orc.mhsa_forward(x.double(), wd, n_heads=H, n_kv_heads=Hkv, qknorm=True, gating="per-head", rope=rope)
     assert torch.allclose(steps.cpu().double(), ref, atol=2e-2, rtol=1e-2)
+
+
+def test_mhsa_module_prefill_with_grad_then_cached_steps_without(gpu_device):
+    """A prefill that runs with gradients enabled (its mixed values are not kept in the cache) followed by
+    generation steps under no_grad: the first cached step mixes every row the cache is still missing, and the value
+    tensor handed on equals the full pass's."""
+    H, Hkv, d, S0, S = 6, 2, 64, 70, 73
+    b, d_model = 1, H * d
+    m, w, rope = _module_and_oracle_weights(gpu_device, BF16, d_model, H, Hkv, True, True, "per-head", seed=19)
+    xd = torch.randn(b, S, d_model, generator=torch.Generator().manual_seed(21)).to(BF16).to(gpu_device)
+    with torch.no_grad():
+        full, V_full = m(xd)
+    cache = KVCache()
+    outs = [m(xd[:, :S0], kv_cache=cache)[0].detach()]  # grad mode on: the module's parameters require grad
+    assert cache.mixed_length == 0
+    with torch.no_grad():
+        for t in range(S0, S):
+            o, V_t = m(xd[:, t : t + 1], kv_cache=cache)
+            outs.append(o)
+            assert cache.mixed_length == t + 1
+    assert torch.allclose(torch.cat(outs, dim=1).float(), full.float(), atol=2e-2, rtol=1e-2)
+    assert torch.allclose(V_t.float(), V_full.float(), atol=1e-2, rtol=1e-2)
+    with pytest.raises(ValueError):
+        cache.append_mixed(V_t[:, :, :2])
 
 
 # ------------------------------------------------------------------ HIP graph capture of a forward + backward pair
