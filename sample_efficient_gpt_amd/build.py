@@ -67,6 +67,15 @@ def build(verbose: bool = False, extra_flags: list[str] | None = None) -> str:
     os.replace(tmp, LIB_PATH)
     if verbose:
         print("built", LIB_PATH)
+    # stand-alone measurement programs (not part of the library): one executable per source under csrc/microbench
+    mb_dir = os.path.join(CSRC, "microbench")
+    for src in sorted(f for f in os.listdir(mb_dir) if f.endswith(".hip")):
+        exe = os.path.join(PKG_DIR, src.replace(".hip", ".bin"))
+        _run([hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+              "-Wno-unused-command-line-argument", os.path.join(mb_dir, src), "-o", exe + ".tmp"])
+        os.replace(exe + ".tmp", exe)
+        if verbose:
+            print("built", exe)
     return LIB_PATH
 
 
