@@ -131,3 +131,52 @@ def compare(got, ref, dtype, names=None, label="", scales=None, outliers=None):
                             f"(ref max {float(r.abs().max()):.3e})")
     assert not failures, "; ".join(failures)
     return errs
+
+
+def bf16_round(t):
+    """Round-to-nearest-even to bf16, kept in the tensor's own (float64) dtype."""
+    return t.to(torch.float32).to(torch.bfloat16).to(t.dtype)
+
+
+def kernel_rounding_model(Q, K, V, g, dO, *, eps, sm_scale, causal, q_start):
+    """The bf16 kernels' mathematics in float64 with a bf16 rounding at every point where the kernels hold a bf16
+    value (csrc/fwd_mfma.hip, bwd_mfma.hip: the normalised operands Qhat and Khat, the probabilities and dS as MFMA
+    operands, the saved output that delta is taken from) and exact arithmetic everywhere else.  Q [n,Sq,D], K, V
+    [n,Sk,D], dO [n,Sq,D] hold bf16 values; g is the combined scale (1 or D elements).  Not a second oracle: it exists
+    to say, per case, how far bf16 operand rounding moves the results away from the exact mathematics (the oracle), so
+    that a test can demand the ordinary tolerance against THIS and report the distance to the oracle separately."""
+    Q, K, V, dO, g = (t.double() for t in (Q, K, V, dO, g))
+    n, Sq, D = Q.shape
+    Sk = K.shape[1]
+    log2e, ln2 = 1.4426950408889634, 0.6931471805599453
+    a = torch.rsqrt((Q * Q).mean(-1, keepdim=True) + eps)
+    b = torch.rsqrt((K * K).mean(-1, keepdim=True) + eps)
+    qhat = bf16_round(sm_scale * log2e * a * Q * g)
+    khat = bf16_round(b * K)
+    s2 = qhat @ khat.transpose(1, 2)  # log2 units
+    if causal:
+        i = torch.arange(Sq).unsqueeze(1)
+        j = torch.arange(Sk).unsqueeze(0)
+        s2 = s2.masked_fill(j > i + q_start, float("-inf"))
+    m = s2.max(-1, keepdim=True).values
+    p = bf16_round(torch.exp2(s2 - m))
+    l = p.sum(-1, keepdim=True)
+    y = bf16_round((p @ V) / l)
+    lse2 = m + torch.log2(l)
+    # backward: P from the saved lse, delta from the saved (rounded) output
+    P = torch.exp2(s2 - lse2)
+    delta = (dO * y).sum(-1, keepdim=True)
+    dP = dO @ V.transpose(1, 2)
+    dS = P * (dP - delta)
+    dv = bf16_round(P).transpose(1, 2) @ dO
+    dSr = bf16_round(dS)
+    T = dSr @ khat                      # dL/dQhat in units of the log2-scaled logits times ln2 ... see below
+    dKhat = dSr.transpose(1, 2) @ qhat  # carries Qhat's sm_scale * log2e * g
+    # dS is the gradient with respect to the NATURAL logit s = ln2 * s2, and s2 = qhat . khat, so
+    # dL/dqhat = ln2 * dS khat and dL/dkhat = ln2 * dS^T qhat; qhat = f a q g with f = sm_scale * log2e
+    u = (ln2 * sm_scale * log2e) * g * T                      # dL/d(a q)
+    dq = a * (u - (a * a / D) * (u * Q).sum(-1, keepdim=True) * Q)
+    dg = ((ln2 * sm_scale * log2e) * T * a * Q).sum((0, 1))  # per dimension; a scalar gain takes its sum
+    W = ln2 * dKhat                                           # dL/dkhat
+    dk = b * W - (b ** 3 / D) * (W * K).sum(-1, keepdim=True) * K
+    return {"y": y, "dq": dq, "dk": dk, "dv": dv, "dg": dg}

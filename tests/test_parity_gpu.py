@@ -269,7 +269,8 @@ def test_full_size_exact_properties(gpu_device, cfg):
 
 
 def test_cfg4_long_context_extras_full_size(gpu_device):
-    _slice_check(gpu_device, CONFIGS[4], [(1, 3)], odtype=torch.float32)
+    # both batches, the first and a later kv group
+    _slice_check(gpu_device, CONFIGS[4], [(0, 0), (1, 3)], odtype=torch.float32)
 
 
 def test_cfg5_wide_head_full_size(gpu_device):
@@ -719,10 +720,10 @@ def test_cpu_patch_formula_variant_c(gpu_device, dtype, S, Sk, q_start, causal):
     logits are gain*d*cos, up to +-64 at head_dim 64) is the family at (eps, sm_scale) = (1e-8, 1): the HIP kernels with
     those parameters against `cpu_patch_variant_c`, forward and every gradient, q_start and non-causal included.
     fp32 at 1e-5.  The logit bound leaves the raw-exponent range, so the bf16 forward takes its running-maximum
-    path; a bf16 logit carries the 2^-9 rounding of both normalised operands times its magnitude, sqrt(d) = 8 times
-    the live module's, so the absolute part of the bf16 tolerance is scaled by 8 after the fp32 kernels have met
-    1e-5 on the same inputs, and so is the relative part (a logit error of 2^-8 * |logit| is a RELATIVE error of exp(logit):
-    up to 8 times the live module's); both norm-wise.  The reference itself runs this formula on the CPU in fp32 only."""
+    path.  A bf16 logit carries the 2^-9 rounding of both normalised operands times its magnitude, sqrt(d) = 8 times
+    the live module's, which no kernel working on bf16 operands can avoid; the bf16 leg therefore compares with a
+    float64 model of the kernels' mathematics that rounds where they round (pinned to the oracle with the roundings
+    switched off) at the ordinary bf16 tolerance.  The reference itself runs this formula on the CPU in fp32 only."""
     D, n = 64, 3
     x = gen(n, 1, 1, S, Sk, D, dtype, no_gk=True, seed=23)
     gain = torch.tensor([1.0])
@@ -760,7 +761,38 @@ def test_cpu_patch_formula_variant_c(gpu_device, dtype, S, Sk, q_start, causal):
     # and the gradients sum thousands of such terms against entries of size 20.
     check(run(F32), 1e-5, 1e-5, "fp32")
     if dtype == BF16:
-        check(run(BF16), 8 * 2e-2, 8 * 1e-2, "bf16")
+        # bf16: the comparison target is derived per case.  `kernel_rounding_model` is the same mathematics in float64 with
+        # a bf16 rounding wherever the kernels hold a bf16 value; with the roundings switched off it must BE the oracle
+        # (that pins it), with them on the kernels have to meet the ORDINARY bf16 tolerance against it, and its own
+        # distance to the oracle, i.e. what operand rounding costs at logits of +-64, is reported (it is what the
+        # earlier blanket allowance of 8x stood for).
+        import tests.parity_util as pu
+
+        args = (Q, K, V, gain.double(), dO)
+        kw = dict(eps=eps, sm_scale=sc, causal=causal, q_start=q_start)
+        keep = pu.bf16_round
+        try:
+            pu.bf16_round = lambda t: t
+            exact = pu.kernel_rounding_model(*args, **kw)
+        finally:
+            pu.bf16_round = keep
+        for name in ("y", "dq", "dk", "dv"):
+            assert float((exact[name] - ref[name]).abs().max()) <= 1e-9 * max(1.0, float(ref[name].abs().max())), name
+        assert abs(float(exact["dg"].sum() - ref["dg_q"])) <= 1e-9 * max(1.0, dgs)
+        model = pu.kernel_rounding_model(*args, **kw)
+        model["dg_q"] = model.pop("dg").sum().reshape(ref["dg_q"].shape)
+        got = run(BF16)
+        for name, r in model.items():
+            g = got[name].double().reshape(r.shape)
+            err = (g - r).abs()
+            # y and dv element-wise; dq, dk norm-wise like the fp32 leg above: delta is taken from the bf16-rounded
+            # output, whose rounding residue (modelled in size, not entry by entry) enters them times the logit scale
+            scale = max(float(r.abs().max()), dgs) if name == "dg_q" else (r.abs() if name in ("y", "dv") else float(r.abs().max()))
+            drift = float((r - ref[name]).abs().max())
+            print(f"  bf16 {name}: max abs err vs the rounding model {float(err.max()):.2e}; the model is {drift:.2e} from the oracle "
+                  f"(largest entry {float(ref[name].abs().max()):.2e})", flush=True)
+            assert bool((err <= 2e-2 + 1e-2 * scale).all()), f"bf16 {name}: max abs err {float(err.max()):.3e} vs the rounding model"
+            assert drift <= 8 * (2e-2 + 1e-2 * float(ref[name].abs().max())), name  # operand rounding stays what it was known to be
 
 
 def test_module_state_dict_and_forward(gpu_device):
