@@ -58,11 +58,16 @@ constexpr float kLazyThresh = 16.f;   // general path: the subtracted reference 
 // NARROW).  NARROW: 32 rows per wave, three stages (48 KB), three workgroups per CU: twice as many, lighter
 // workgroups whose start-up / write-out latencies hide behind two neighbours instead of one (S = 2048: 1 %
 // faster, S = 1152: 10 %, S = 768: 13 %, S = 384: 27 %).  The launcher picks by the number of keys.
+// head_dim 128: 32 rows per wave and 32-KEY tiles (a tile pair is then the same 16 KB as at head_dim 64, a block of a
+// tile carries twice the MFMAs, so one block per tile keeps the ratio of barriers and tile loads to MFMAs), four stages
+// = 64 KB, two workgroups per CU.  With 64-key tiles the ring alone is 96 KB and a CU holds one workgroup, i.e. one
+// wave per SIMD with nothing to overlap its softmax phase with.
 template <int D, bool WIDE>
 struct FwdShape {
   static constexpr int kNQB = (D == 64 && WIDE) ? 2 : 1;  // 32-query blocks per wave
-  static constexpr int kStages = D == 64 ? (WIDE ? 4 : 3) : 3;
-  static constexpr int kOcc = D == 64 ? (WIDE ? 2 : 3) : 1;
+  static constexpr int kBK = D == 64 ? 64 : 32;           // keys per streamed tile
+  static constexpr int kStages = D == 64 ? (WIDE ? 4 : 3) : 4;
+  static constexpr int kOcc = D == 64 ? (WIDE ? 2 : 3) : 2;
   static constexpr int kBQ = 4 * 32 * kNQB;
 };
 
@@ -70,9 +75,10 @@ struct FwdShape {
 // travel with the start-up tiles instead of costing a memory round trip of their own behind a branch.
 template <int D, bool WIDE, bool ROPE>
 __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16_kernel(KArgs a) {
-  using Z = Swz<D>;
   using F = FwdShape<D, WIDE>;
-  constexpr int NQB = F::kNQB, BQ = F::kBQ, NS = F::kStages;
+  constexpr int NQB = F::kNQB, BQ = F::kBQ, NS = F::kStages, BK = F::kBK;
+  constexpr int kBlocksPerTile = BK / 32;
+  using Z = Swz<D, BK>;
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
   constexpr int kStageBytes = 2 * Z::kTileBytes;
@@ -94,7 +100,7 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
 
   int kend = p.Sk;
   if (p.causal) kend = min(p.Sk, q0 + BQ + p.q_start);
-  const int n_kt = (kend + kBK - 1) / kBK;
+  const int n_kt = (kend + BK - 1) / BK;
   const char* kbase = reinterpret_cast<const char*>(a.khat + ((int64_t)b * p.Hkv + g) * p.Sk * D);
   const char* vbase = a.vmix ? reinterpret_cast<const char*>(a.vmix + ((int64_t)b * p.Hkv + g) * p.Sk * D)
                              : reinterpret_cast<const char*>(row_ptr<uint16_t>(p.v, b, g, 0));
@@ -103,14 +109,14 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
   const uint32_t lds0 = lds_addr_of(lds);
   const int2 src = swz_src<D>(lane, wave);
   const uint32_t wave_dst = lds0 + wave * 1024;
-  const TileLaneOff<D> full_tile = tile_lane_offsets<D>(kstep, vstep, kBK, src.x, src.y);
+  const TileLaneOff<D, BK> full_tile = tile_lane_offsets<D, BK>(kstep, vstep, BK, src.x, src.y);
   auto issue_tile = [&](int jt) {  // tile jt -> stage jt % NS
-    const char* ksrc = kbase + (int64_t)jt * kBK * kstep;
-    const char* vsrc = vbase + (int64_t)jt * kBK * vstep;
+    const char* ksrc = kbase + (int64_t)jt * BK * kstep;
+    const char* vsrc = vbase + (int64_t)jt * BK * vstep;
     const uint32_t dst = wave_dst + (jt % NS) * kStageBytes;
-    const int left = p.Sk - jt * kBK;
-    if (left >= kBK) issue_tile_pair<D>(ksrc, vsrc, full_tile, dst);
-    else issue_tile_pair<D>(ksrc, vsrc, tile_lane_offsets<D>(kstep, vstep, left, src.x, src.y), dst);
+    const int left = p.Sk - jt * BK;
+    if (left >= BK) issue_tile_pair<D, BK>(ksrc, vsrc, full_tile, dst);
+    else issue_tile_pair<D, BK>(ksrc, vsrc, tile_lane_offsets<D, BK>(kstep, vstep, left, src.x, src.y), dst);
   };
 
   // ---- start-up.  The workgroup's query rows come in as tiles too (read row-per-lane from global memory, every
@@ -119,7 +125,7 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
   // kQStages stages of the ring, the first kEarlyTiles key tiles (those that fit before them) are requested at the
   // same time, the scale vector behind them: one memory round trip.  The remaining start-up tiles follow once the
   // query rows sit in registers (run() below).
-  constexpr int kQStages = BQ / 128;            // 128 rows (two tiles) per stage
+  constexpr int kQStages = BQ / (2 * BK);       // a stage holds two tiles of BK rows
   constexpr ring::Protocol R = ring::forward(NS, kQStages, Z::kPasses);  // the pipeline's numbers: ring_protocol.hpp
   static_assert(ring::well_formed(R) && R.loads_per_tile == kLoadsPerTile && !R.wait_before_loop && R.issue_at_top, "tile pipeline");
   static_assert(R.early_tiles >= ring::kTilesNeededAtLoopStart, "the loop is entered without a further wait");
@@ -130,7 +136,7 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
     const char* qb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.q, b, h, q0));
 #pragma unroll
     for (int i = 0; i < kQStages; ++i)
-      issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, 128 * i, p.Sq - q0, src.x, src.y),
+      issue_tile_pair<D, BK>(qb, qb, rowblock_lane_offsets<D, BK>((uint32_t)p.q.stride_s * 2, 2 * BK * i, p.Sq - q0, src.x, src.y),
                          wave_dst + (R.row_stage_first + i) * kStageBytes);
   }
 
@@ -153,8 +159,8 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
 #pragma unroll
   for (int nb = 0; nb < NQB; ++nb) {
     const int row = min(qw0 + 32 * nb + ln, p.Sq - 1);
-    // rows 32*(NQB*wave + nb) .. +31 of the block: 64-row tile (that / 2), row block (that & 1)
-    const int blk = NQB * wave + nb, tile = blk >> 1, rb = blk & 1;
+    // rows 32*(NQB*wave + nb) .. +31 of the block: which BK-row tile of the staged block, and which 32-row block of it
+    const int blk = NQB * wave + nb, tile = blk / kBlocksPerTile, rb = blk % kBlocksPerTile;
     const uint32_t rm = lds0 + (R.row_stage_first + (tile >> 1)) * kStageBytes + (tile & 1) * Z::kTileBytes + swz_off_rm<D>(lane);
     u32x4 raw[KS];
 #pragma unroll
@@ -301,15 +307,19 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
     // Two loops instead of a per-block choice inside one: each body is then a single straight-line region
     // with one variant of the block (a join of the two variants costs a copy of every accumulator).
     // Loop A: tiles whose two blocks need no mask.  Loop B: the rest (masking a fully visible block is a no-op).
-    const int n_a = n_full / 2;  // n_full <= n_act, so these tiles are all active
+    const int n_a = n_full / kBlocksPerTile;  // n_full <= n_act, so these tiles are all active
     int jt = 0;
     for (; jt < n_a; ++jt) {
       const int nstage = stage == NS - 1 ? 0 : stage + 1;
       const bool issued = jt + R.issue_ahead < n_kt;
       if (issued) issue_tile(jt + R.issue_ahead);
       const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
-      step(IC<0>{}, bounded_c, tr, 0, 64 * jt, rm, 1);
-      step(IC<0>{}, bounded_c, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
+      if constexpr (kBlocksPerTile == 2) {
+        step(IC<0>{}, bounded_c, tr, 0, BK * jt, rm, 1);
+        step(IC<0>{}, bounded_c, tr, 1, BK * jt + 32, rm_lane + nstage * kStageBytes, 0);
+      } else {
+        step(IC<0>{}, bounded_c, tr, 0, BK * jt, rm_lane + nstage * kStageBytes, 0);
+      }
       if (issued) wait_vmcnt<ring::loads_kept_after_iteration(R, true)>(); else wait_vmcnt<ring::loads_kept_after_iteration(R, false)>();
       __syncthreads();
       stage = nstage;
@@ -319,8 +329,12 @@ __global__ __launch_bounds__(kThreadsM, (FwdShape<D, WIDE>::kOcc)) void fwd_bf16
       const bool issued = jt + R.issue_ahead < n_kt;
       if (issued) issue_tile(jt + R.issue_ahead);
       const uint32_t rm = rm_lane + stage * kStageBytes, tr = tr_lane + stage * kStageBytes;
-      if (2 * jt < n_act) step(IC<1>{}, bounded_c, tr, 0, 64 * jt, rm, 1);
-      if (2 * jt + 1 < n_act) step(IC<1>{}, bounded_c, tr, 1, 64 * jt + 32, rm_lane + nstage * kStageBytes, 0);
+      if constexpr (kBlocksPerTile == 2) {
+        if (2 * jt < n_act) step(IC<1>{}, bounded_c, tr, 0, BK * jt, rm, 1);
+        if (2 * jt + 1 < n_act) step(IC<1>{}, bounded_c, tr, 1, BK * jt + 32, rm_lane + nstage * kStageBytes, 0);
+      } else {
+        if (jt < n_act) step(IC<1>{}, bounded_c, tr, 0, BK * jt, rm_lane + nstage * kStageBytes, 0);
+      }
       if (issued) wait_vmcnt<ring::loads_kept_after_iteration(R, true)>(); else wait_vmcnt<ring::loads_kept_after_iteration(R, false)>();
       __syncthreads();
       stage = nstage;

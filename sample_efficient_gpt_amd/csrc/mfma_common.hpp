@@ -69,10 +69,11 @@ __device__ __forceinline__ u32x4 scale8(u32x4 v, float f) {
 //   D = 64  (8 chunks / row):   f(r) = (r >> 1) & 7
 //   D = 128 (16 chunks / row):  f(r) = ((r & 3) << 2) | ((r >> 2) & 3)
 // Both depend on r mod 16 only and satisfy f(r + 8) = f(r) ^ kHiXorChunks for r < 8.
-template <int D>
+template <int D, int ROWS = kBK>
 struct Swz {
+  static constexpr int kRows = ROWS;                    // rows per tile (64; the head_dim-128 forward streams 32-row tiles)
   static constexpr int kRB = 2 * D;                     // bytes per row
-  static constexpr int kTileBytes = kBK * kRB;          // 8 KB (D=64) / 16 KB (D=128)
+  static constexpr int kTileBytes = ROWS * kRB;         // 8 KB (D=64, or D=128 with 32 rows) / 16 KB (D=128)
   static constexpr int kChunks = kRB / 16;              // chunks per row
   static constexpr int kRowsPerInst = 1024 / kRB;       // rows one wave-wide load covers
   static constexpr int kPasses = kTileBytes / 1024 / 4; // wave-wide loads per wave per tile (4 waves)
@@ -81,6 +82,7 @@ struct Swz {
     return D == 64 ? ((row >> 1) & 7) : (((row & 3) << 2) | ((row >> 2) & 3));
   }
   static_assert(D == 64 || D == 128, "swizzle is defined for 128- and 256-byte rows");
+  static_assert(kPasses >= 1 && kPasses * 4 * kRowsPerInst == ROWS, "four waves fill a tile in whole passes");
 };
 
 // s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt = {imm[15:14], imm[3:0]}, expcnt / lgkmcnt left at max)
@@ -347,14 +349,14 @@ __device__ __forceinline__ f32x16 splat16(float x) {
 // computed once (rows_left = 64) and a tile then costs no vector arithmetic; a last, partial tile gets its own
 // set, in which rows past rows_left re-read the last valid row (callers mask them).
 //   step_*: bytes between rows; lane_row / lane_col: from swz_src()
-template <int D>
+template <int D, int ROWS = kBK>
 struct TileLaneOff {
-  uint32_t a[Swz<D>::kPasses], b[Swz<D>::kPasses];
+  uint32_t a[Swz<D, ROWS>::kPasses], b[Swz<D, ROWS>::kPasses];
 };
-template <int D>
-__device__ __forceinline__ TileLaneOff<D> tile_lane_offsets(uint32_t step_a, uint32_t step_b, int rows_left, int lane_row, int lane_col) {
-  using Z = Swz<D>;
-  TileLaneOff<D> o;
+template <int D, int ROWS = kBK>
+__device__ __forceinline__ TileLaneOff<D, ROWS> tile_lane_offsets(uint32_t step_a, uint32_t step_b, int rows_left, int lane_row, int lane_col) {
+  using Z = Swz<D, ROWS>;
+  TileLaneOff<D, ROWS> o;
 #pragma unroll
   for (int ps = 0; ps < Z::kPasses; ++ps) {
     const int row = min(lane_row + ps * 4 * Z::kRowsPerInst, rows_left - 1);
@@ -363,18 +365,18 @@ __device__ __forceinline__ TileLaneOff<D> tile_lane_offsets(uint32_t step_a, uin
   }
   return o;
 }
-// The same for 128 rows of ONE tensor, staged as the two tiles of a stage: a = rows row_first .. +63, b = rows
-// row_first+64 .. +127, both as offsets from the tensor block's first row (row 0, of which rows_left >= 1 exist;
+// The same for 2*ROWS rows of ONE tensor, staged as the two tiles of a stage: a = rows row_first .. +ROWS-1, b = the
+// ROWS rows after them, both as offsets from the tensor block's first row (row 0, of which rows_left >= 1 exist;
 // later rows re-read the last one), so the rows are issued as issue_tile_pair(base, base, offsets, stage).
-template <int D>
-__device__ __forceinline__ TileLaneOff<D> rowblock_lane_offsets(uint32_t step, int row_first, int rows_left, int lane_row, int lane_col) {
-  using Z = Swz<D>;
-  TileLaneOff<D> o;
+template <int D, int ROWS = kBK>
+__device__ __forceinline__ TileLaneOff<D, ROWS> rowblock_lane_offsets(uint32_t step, int row_first, int rows_left, int lane_row, int lane_col) {
+  using Z = Swz<D, ROWS>;
+  TileLaneOff<D, ROWS> o;
 #pragma unroll
   for (int ps = 0; ps < Z::kPasses; ++ps) {
     const int r = row_first + lane_row + ps * 4 * Z::kRowsPerInst;
     o.a[ps] = (uint32_t)min(r, rows_left - 1) * step + lane_col;
-    o.b[ps] = (uint32_t)min(r + kBK, rows_left - 1) * step + lane_col;
+    o.b[ps] = (uint32_t)min(r + ROWS, rows_left - 1) * step + lane_col;
   }
   return o;
 }
@@ -389,9 +391,9 @@ __device__ __forceinline__ u32x2 lds_read8(uint32_t addr) {
   return *(const __attribute__((address_space(3))) u32x2*)addr;
 }
 //   src_a/src_b: wave-uniform pointers to row `row0` of each tensor; dst: LDS byte address of the stage + wave*1024
-template <int D>
-__device__ __forceinline__ void issue_tile_pair(const char* src_a, const char* src_b, const TileLaneOff<D>& o, uint32_t dst) {
-  using Z = Swz<D>;
+template <int D, int ROWS = kBK>
+__device__ __forceinline__ void issue_tile_pair(const char* src_a, const char* src_b, const TileLaneOff<D, ROWS>& o, uint32_t dst) {
+  using Z = Swz<D, ROWS>;
 #pragma unroll
   for (int ps = 0; ps < Z::kPasses; ++ps) {
     gload_lds16_so(src_a, o.a[ps], dst + ps * 4096);
