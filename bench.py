@@ -139,7 +139,9 @@ def cpu_baseline(c, batches: int, budget_s: float = 12.0):
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
         "host_cores": host_cores,
-        "parallel_info": torch.__config__.parallel_info().strip().splitlines()[0],
+        # the informative lines of torch.__config__.parallel_info(): thread counts and the threading backend
+        "parallel_info": " | ".join(l.strip() for l in torch.__config__.parallel_info().splitlines()
+                                    if any(k in l for k in ("get_num_threads", "omp_get_max_threads", "ATen parallel backend"))),
         "kind": "port",
         "sample": f"{passes} passes over {batches} of {c.B} batches of the same workload, fp32, fwd{'+bwd' if c.backward else ''} "
                   f"({dt:.1f} s in all): RMS-normalise + F.scaled_dot_product_attention(is_causal) + autograd",
