@@ -62,6 +62,12 @@ KvLayout kv_layout(const segpt_attn_params& p) {
   return w;
 }
 
+// The backward keeps a gate-scaled copy of dO on the fp32 path and, on the bf16 path, only for a gate scale that is
+// not positive: a positive gate factor travels to the dK/dV kernel inside the two row statistics instead.
+bool gated_do_copy(const segpt_attn_params& p) {
+  return p.gate.ptr && (p.dtype == SEGPT_DTYPE_FP32 || !(p.gate_scale > 0.f));
+}
+
 WsLayout bwd_layout(const segpt_attn_params& p) {
   WsLayout w;
   size_t off = 0;
@@ -71,7 +77,7 @@ WsLayout bwd_layout(const segpt_attn_params& p) {
   w.nlse2 = off;
   if (p.dtype == SEGPT_DTYPE_BF16) off += align_up(rows * sizeof(float));
   w.do_eff = off;
-  if (p.gate.ptr) off += align_up(rows * p.D * elem_bytes(p));
+  if (gated_do_copy(p)) off += align_up(rows * p.D * elem_bytes(p));
   w.qhat = off;
   if (p.dtype == SEGPT_DTYPE_BF16) off += align_up(rows * p.D * 2);
   w.dg_part = off;
@@ -317,7 +323,7 @@ static int bwd_stage_impl(const segpt_attn_params* p_in, int stage_lo, int stage
   a.p = *p;
   char* ws = reinterpret_cast<char*>(p->workspace);
   a.delta = reinterpret_cast<float*>(ws + w.delta);
-  a.do_eff = p->gate.ptr ? ws + w.do_eff : nullptr;
+  a.do_eff = gated_do_copy(*p) ? ws + w.do_eff : nullptr;
   a.dg_part = reinterpret_cast<float*>(ws + w.dg_part);
   a.dcoef_part = reinterpret_cast<float*>(ws + w.dcoef_part);
   if (p->dtype == SEGPT_DTYPE_BF16) {

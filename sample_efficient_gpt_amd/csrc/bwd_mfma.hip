@@ -2,8 +2,8 @@
 //
 // Operands are normalised tensors held in the workspace (bf16):
 //   Khat = b_j k_j and V' = c1 v + c2 v_first, written by the key/value pre-pass (pre_post.hip);
-//   Qhat = sm_scale*log2e * a_i q_i * g_q*g_k, delta and the gate-scaled dO, written by the dQ kernel's
-//   prologue for the dK/dV kernel that runs after it.
+//   Qhat = sm_scale*log2e * a_i q_i * g_q*g_k and the two row statistics -lse2, -delta (which also carry a positive
+//   gate factor), written by the dQ kernel for the dK/dV kernel that runs after it.
 //
 //  bwd_dq    query-stationary, same orientation as the forward (a lane owns one query column):
 //              S^T  = Khat . Qhat^T - lse2        dP^T = V' . dO^T - delta     (A from LDS row-major,
@@ -32,11 +32,13 @@ constexpr int kBwdRows = 4 * 32;  // rows (queries for dQ, keys for dK/dV) owned
 // was measured 13 % slower at B*Hkv = 12, S = 8192 (where forward and dQ gain 2-4 % from pinning 8 of the 12).
 __host__ __device__ inline int dkdv_pinned(const segpt_attn_params& p) { return wg_pinned_pairs(p.B, p.Hkv, true); }
 
+constexpr float kGateFactorFloor = 1e-30f;  // a smaller gate factor switches its row off in the dK/dV kernel
+
 constexpr int kStages = 4;  // LDS ring of streamed stages (two tiles each): tile t lives in stage t % 4
 
 // ============================================================================================ dQ
 // Also the producer of the per-query-row quantities the dK/dV kernel streams afterwards: Qhat, -delta,
-// -lse*log2e and (with a gate) the gate-scaled dO and dgate.
+// -lse*log2e and (with a gate) dgate; the gate-scaled copy of dO only when the gate scale is not positive.
 //
 // Software pipeline over 32-key blocks n (two per staged tile), one barrier per tile:
 //   B(n)  S^T, dP^T MFMAs from the row-major fragments requested one block earlier
@@ -167,7 +169,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
 
   // ---- query-row prologue: alpha, Qhat, delta, gate; B operands stay in registers
   bf16x8 qreg[KS], doreg[KS];
-  float alpha, delta, dgate_row = 0.f;
+  float alpha, delta, dgate_row = 0.f, gfac = 1.f;
   {
     float dl = 0.f;
 #pragma unroll
@@ -186,7 +188,6 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     delta = half_sum(dl);
     alpha = row_normaliser_fast(p, ss, 1.0f / D);
     const float f = alpha * p.sm_scale * kLog2e;
-    float gfac = 1.f;
     if (p.gate.ptr) {
       const float sg = 1.0f / (1.0f + __expf(-gate_z));
       gfac = p.gate_scale * sg;
@@ -300,18 +301,27 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
     stage = nstage;
   }
 
-  // ---- epilogue.  First what the dK/dV kernel reads of this row: Qhat, the gated dO, -delta, -lse2 (and dgate).
+  // ---- epilogue.  First what the dK/dV kernel reads of this row: Qhat, -delta, -lse2 (and dgate).  A gate factor
+  // f > 0 reaches that kernel through the two statistics and it streams the caller's dO as it is: with
+  // P' = f P = exp2(S - lse2 + log2 f) it holds dV' = P'^T dO and dS = P (f dP - delta) = P' (dP - delta / f).  A
+  // factor that underflowed switches the row off (P' = 0).  Only a gate scale <= 0 needs the gated copy of dO.
   RopeCt<MB> rope_ct;
   if (ROPE) rope_ct = rope_ct_load<MB>(p.rope_cos + rope_pos, p.rope_sin + rope_pos, hh);
   if (live) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       *reinterpret_cast<bf16x8*>(a.qhat + ridx * D + 16 * ks + 8 * hh) = qreg[ks];
-      if (p.gate.ptr) *reinterpret_cast<bf16x8*>(reinterpret_cast<uint16_t*>(a.do_eff) + ridx * D + 16 * ks + 8 * hh) = doreg[ks];
+      if (a.do_eff) *reinterpret_cast<bf16x8*>(reinterpret_cast<uint16_t*>(a.do_eff) + ridx * D + 16 * ks + 8 * hh) = doreg[ks];
     }
     if (hh == 0) {
-      a.delta[ridx] = -delta;
-      a.nlse2[ridx] = nlse2;
+      float stat_d = -delta, stat_l = nlse2;
+      if (p.gate.ptr && !a.do_eff) {
+        const bool on = gfac > kGateFactorFloor;
+        stat_l = on ? nlse2 + __log2f(gfac) : -INFINITY;
+        stat_d = on ? -delta / gfac : 0.f;
+      }
+      a.delta[ridx] = stat_d;
+      a.nlse2[ridx] = stat_l;
       if (p.gate.ptr)
         reinterpret_cast<uint16_t*>(p.dgate.ptr)[(int64_t)b * p.dgate.stride_b + (int64_t)row * p.dgate.stride_s + (int64_t)h * p.dgate.stride_h] = f32_to_bf16(dgate_row);
     }

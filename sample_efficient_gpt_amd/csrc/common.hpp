@@ -16,7 +16,7 @@ struct KArgs {
   segpt_attn_params p;
   float* delta;       // [B,H,Sq] fp32: rowsum(dO_eff * o)  (fp32 path) / its NEGATIVE (bf16 path: MFMA C operand)
   float* nlse2;       // [B,H,Sq] fp32: -lse*log2(e)                 (bf16 path only: MFMA C operand)
-  void* do_eff;       // [B,H,Sq,D] dtype, contiguous: gate-scaled dO (only when gated)
+  void* do_eff;       // [B,H,Sq,D] dtype, contiguous: gate-scaled dO (fp32 path; bf16 path only for a gate scale <= 0), else null
   uint16_t* qhat;     // [B,H,Sq,D]   bf16: sm_scale*log2e * a_i q_i * g_q*g_k   (bf16 path only)
   uint16_t* khat;     // [B,Hkv,Sk,D] bf16: b_j k_j                               (bf16 path only; kv_workspace)
   uint16_t* vmix;     // [B,Hkv,Sk,D] bf16: c1 v + c2 v_first (only with a value residual, else NULL; kv_workspace)

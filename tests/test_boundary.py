@@ -164,7 +164,13 @@ def test_workspace_bytes(lib):
     rows = 2 * 6 * 128
     assert base >= rows * 4 and base % 256 == 0
     p.gate = _lib.Tensor3(0x10000, 128 * 6, 6, 1)
-    assert lib.segpt_attn_workspace_bytes(p, 1) >= base + rows * 64 * 2  # + gated dO copy
+    assert lib.segpt_attn_workspace_bytes(p, 1) == base  # gate scale 2: the gate factor travels in the row statistics
+    p.gate_scale = -1.0
+    assert lib.segpt_attn_workspace_bytes(p, 1) == base + rows * 64 * 2  # a gate scale <= 0: + gated dO copy
+    p32 = _valid_params(dtype=_lib.SEGPT_DTYPE_FP32)
+    base32 = lib.segpt_attn_workspace_bytes(p32, 1)
+    p32.gate = _lib.Tensor3(0x10000, 128 * 6, 6, 1)
+    assert lib.segpt_attn_workspace_bytes(p32, 1) == base32 + rows * 64 * 4  # fp32 path: always
     bad = _valid_params(); bad.struct_bytes = 4
     assert lib.segpt_attn_workspace_bytes(bad, 1) == 0
 

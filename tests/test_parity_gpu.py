@@ -17,8 +17,8 @@ pytestmark = pytest.mark.gpu
 BF16, F32 = torch.bfloat16, torch.float32
 
 
-def _case(device, dtype, B, H, Hkv, Sq, Sk, D, *, backward=True, seed=0, gen_kw=None, outliers=None, **kw):
-    x = gen(B, H, Hkv, Sq, Sk, D, dtype, seed=seed, **(gen_kw or {}))
+def _case(device, dtype, B, H, Hkv, Sq, Sk, D, *, backward=True, seed=0, gen_kw=None, outliers=None, _x=None, **kw):
+    x = gen(B, H, Hkv, Sq, Sk, D, dtype, seed=seed, **(gen_kw or {})) if _x is None else _x
     print(f"case dtype={dtype} B={B} H={H} Hkv={Hkv} Sq={Sq} Sk={Sk} D={D} bwd={backward} gen={gen_kw} "
           f"kw={ {k: v for k, v in kw.items() if k != 'rope'} } rope={'rope' in kw}", flush=True)
     got = run_gpu(x, device, backward=backward, **kw)
@@ -121,6 +121,47 @@ def test_bf16_reference_training_contexts(gpu_device, S):
     layout (GQA 3:1, head_dim 64), gate + value residual as the model runs them: 768 and 896 are multiples of the
     128-row workgroup tile, 1152 is nine tiles (an odd count for the paired 64-row stages)."""
     _case(gpu_device, BF16, 2, 6, 2, S, S, 64, seed=S, gen_kw={"extras": True}, gate_scale=2.0)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_bf16_gate_factor_through_the_row_statistics(gpu_device, D):
+    """The dK/dV kernel receives a positive gate factor f inside the two row statistics (-lse2 + log2 f, -delta / f)
+    and streams the caller's dO.  Gate logits over the whole range of the sigmoid: saturated on (f = gate_scale),
+    ordinary, so negative that f is 1e-20 (still carried), and so negative that it underflows (the row is switched
+    off: its contributions to dk, dv, dq, dgate are below 1e-30 in the oracle too)."""
+    x = gen(2, 6, 2, 300, 300, D, BF16, extras=True, seed=5)
+    z = x["gate_logits"]
+    S = z.shape[1]
+    z[:, 0::7] = 30.0
+    z[:, 3::7] = -46.0
+    z[:, 5::7] = -90.0
+    z[:, 6::7] = -200.0
+    z[1, S // 2:] = -200.0  # whole query tiles switched off
+    _case(gpu_device, BF16, 2, 6, 2, 300, 300, D, gate_scale=2.0, _x=x)
+    got = run_gpu(x, gpu_device, gate_scale=2.0)
+    for n, t in got.items():
+        assert torch.isfinite(t.float()).all(), n
+
+
+def test_bf16_gate_scale_not_positive_takes_the_gated_copy(gpu_device):
+    """A gate scale <= 0 has no logarithm: the dQ kernel then leaves a gate-scaled copy of dO for the dK/dV kernel
+    (the workspace grows by that tensor)."""
+    from sample_efficient_gpt_amd import _lib
+    from sample_efficient_gpt_amd.function import _fill_common
+    x = gen(1, 4, 2, 200, 200, 64, BF16, extras=True, seed=6)
+    _case(gpu_device, BF16, 1, 4, 2, 200, 200, 64, gate_scale=-1.5, _x=x)
+    _case(gpu_device, BF16, 1, 4, 2, 200, 200, 64, gate_scale=0.0, _x=x)
+    lib = _lib.load()
+    sizes = {}
+    for gs in (2.0, -1.5):
+        p = _lib.new_params()
+        t = {n: x[n] for n in ("q", "k", "v", "v_first", "gate_logits")}
+        y = torch.empty_like(t["q"])
+        lse = torch.empty(t["q"].shape[:3], dtype=torch.float32)
+        _fill_common(p, t["q"], t["k"], t["v"], y, lse, x["g_q"].float(), x["g_k"].float(), t["v_first"], x["vr_coef"].float(),
+                     t["gate_logits"], gs, 1e-6, 0.125, True, 0)
+        sizes[gs] = lib.segpt_attn_workspace_bytes(p, _lib.SEGPT_WS_BWD)
+    assert sizes[-1.5] - sizes[2.0] == 1 * 4 * 200 * 64 * 2 + (-(1 * 4 * 200 * 64 * 2) % 256), sizes
 
 
 def _slice_inputs(c, x, b, g):
