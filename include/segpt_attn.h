@@ -97,7 +97,9 @@ extern "C" {
                                     Khat (and V' = c1 v + c2 v_first) into kv_workspace;
                                     fp32: delta = rowsum(dY*Y), dgate and the gate-scaled dO            */
 #define SEGPT_BWD_STAGE_DQ 1     /* dQ and the per-workgroup partials of the scale gradient; on the bf16
-                                    path also delta, dgate, Qhat and the gate-scaled dO for stage 2      */
+                                    path also delta, dgate and Qhat for stage 2 (a positive gate factor
+                                    is folded into the row statistics; a gate scale <= 0 adds a
+                                    gate-scaled copy of dO)                                              */
 #define SEGPT_BWD_STAGE_DKDV 2   /* dK, dV (, dV_first, partial sums of d vr_coef); bf16: also dg_q, dg_k from
                                     the partials of stage 1                                              */
 #define SEGPT_BWD_STAGE_REDUCE 3 /* d vr_coef from the partials (fp32: also dg_q, dg_k); launches nothing on
