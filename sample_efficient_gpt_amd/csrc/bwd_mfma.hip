@@ -632,10 +632,48 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
     run_tiles(IC<2>{}, t_end, n_vis);
   }
 
-  // ---- epilogue: lane = key row, registers = head-dim entries
+  // ---- epilogue: lane = key row, registers = head-dim entries.  The rows it reads (the raw key for the normaliser's
+  // gradient, with a value residual the raw v and v_first rows for the coefficient gradients) come in like the
+  // prologue's rows: as 128-row blocks by direct loads into the ring's stages, which are idle now (every wave has
+  // passed the last iteration's barrier), and from there in the accumulators' layout.  Read row-per-lane from global
+  // memory, 8 bytes per lane, every wave-wide load would touch 32 cache lines and the three tensors would keep the
+  // address path of the vector memory unit busy for 4-12 us of the launch.
   const bool live = key < p.Sk;
   float c1 = 1.f, c2 = 0.f;
   if (p.vr_coef) { c1 = p.vr_coef[0]; c2 = p.vr_coef[1]; }
+  u32x2 kraw[MB][4], vraw[MB][4], fraw[MB][4];
+  {
+    const int rows_left = p.Sk - k0;
+    const uint32_t wave_dst = lds0 + wave * 1024;
+    const char* kb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.k, b, g, k0));
+    issue_tile_pair<D>(kb, kb, rowblock_lane_offsets<D>((uint32_t)p.k.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst);
+    if (p.vr_coef) {
+      const char* vb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.v, b, g, k0));
+      const char* fb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.v_first, b, g, k0));
+      issue_tile_pair<D>(vb, vb, rowblock_lane_offsets<D>((uint32_t)p.v.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + kStageBytes);
+      issue_tile_pair<D>(fb, fb, rowblock_lane_offsets<D>((uint32_t)p.v_first.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + 2 * kStageBytes);
+    }
+    wait_vmcnt<0>();
+    __syncthreads();
+    // rows 32*wave .. +31 of a block: half (wave >> 1) of its stage, row block (wave & 1) of that tile
+    const uint32_t ct = lds0 + (wave >> 1) * Z::kTileBytes + swz_off_ct<D>(lane) + (wave & 1) * 32 * Z::kRB;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const uint32_t off = (uint32_t)((4 * mb + c) << 4);
+        kraw[mb][c] = lds_read8(ct ^ off);
+        if (p.vr_coef) {
+          vraw[mb][c] = lds_read8((ct + kStageBytes) ^ off);
+          fraw[mb][c] = lds_read8((ct + 2 * kStageBytes) ^ off);
+        }
+      }
+  }
+  RopeCt<MB> rope_ct;
+  if (ROPE) {
+    const int64_t pos = (int64_t)(p.rope_k_pos0 + key_c) * (D / 2);
+    rope_ct = rope_ct_load<MB>(p.rope_cos + pos, p.rope_sin + pos, hh);
+  }
   {
     uint16_t* ovp = row_ptr_mut<uint16_t>(p.dv, b, g, key_c);
 #pragma unroll
@@ -649,19 +687,17 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   if (p.vr_coef) {
     float s1 = 0.f, s2 = 0.f;
     uint16_t* ofp = row_ptr_mut<uint16_t>(p.dv_first, b, g, key_c);
-    const uint16_t* vp = row_ptr<uint16_t>(p.v, b, g, key_c);
-    const uint16_t* fp = row_ptr<uint16_t>(p.v_first, b, g, key_c);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       float val[16], vv[16], ff[16];
-      load_ct_block(vp, mb, hh, vv);
-      load_ct_block(fp, mb, hh, ff);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        val[r] = c2 * dvacc[mb][r];
-        if (live) { s1 += dvacc[mb][r] * vv[r]; s2 += dvacc[mb][r] * ff[r]; }
-      }
+      for (int r = 0; r < 16; ++r) val[r] = c2 * dvacc[mb][r];
       store_ct_block(ofp, mb, hh, live, val);
+      unpack_ct_block(vraw[mb], vv);
+      unpack_ct_block(fraw[mb], ff);
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (live) { s1 += dvacc[mb][r] * vv[r]; s2 += dvacc[mb][r] * ff[r]; }
     }
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) { s1 += __shfl_xor(s1, o, 64); s2 += __shfl_xor(s2, o, 64); }
@@ -671,16 +707,11 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   }
   // dk through the normaliser: W = ln2 * dkacc = dL/dKhat (natural units), dk = b W - (b^3/D)(W.k) k
   {
-    const uint16_t* kp = row_ptr<uint16_t>(p.k, b, g, key_c);
     float kv[MB][16];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) load_ct_block(kp, mb, hh, kv[mb]);
-    RopeCt<MB> rope_ct;
-    if (ROPE) {  // the normaliser acted on the rotated key: work in that frame, rotate the gradient back
-      const int64_t pos = (int64_t)(p.rope_k_pos0 + key_c) * (D / 2);
-      rope_ct = rope_ct_load<MB>(p.rope_cos + pos, p.rope_sin + pos, hh);
-      rope_ct_apply<MB, false>(kv, rope_ct);
-    }
+    for (int mb = 0; mb < MB; ++mb) unpack_ct_block(kraw[mb], kv[mb]);
+    // the normaliser acted on the rotated key: work in that frame, rotate the gradient back
+    if (ROPE) rope_ct_apply<MB, false>(kv, rope_ct);
     float dot = 0.f, ss = 0.f;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
