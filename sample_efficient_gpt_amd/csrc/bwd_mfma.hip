@@ -57,8 +57,11 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   constexpr int KS = D / 16;
   constexpr int MB = D / 32;
   constexpr int kStageBytes = 2 * Z::kTileBytes;
-  constexpr ring::Protocol R = ring::dq(Z::kPasses);  // the pipeline's numbers: ring_protocol.hpp
-  static_assert(ring::well_formed(R) && R.stages == kStages && R.row_stages == 3 && R.wait_before_loop && !R.issue_at_top, "tile pipeline");
+  // the pipeline's numbers: ring_protocol.hpp
+  constexpr ring::Protocol R = ROPE ? ring::dq_rope(Z::kPasses) : ring::dq(Z::kPasses);
+  static_assert(ring::well_formed(R) && R.stages == kStages && !R.issue_at_top, "tile pipeline");
+  static_assert(ROPE ? (R.pre_row_stages == 4 && R.row_stages == 1 && R.early_tiles == R.startup_tiles && !R.wait_before_loop && R.epilogue_row_stages == 2)
+                     : (R.pre_row_stages == 0 && R.row_stages == 3 && R.wait_before_loop && R.epilogue_row_stages == 0), "tile pipeline");
   const segpt_attn_params& p = a.p;
   __shared__ __attribute__((aligned(1024))) char lds[kStages * kStageBytes];
   __shared__ __attribute__((aligned(16))) float gsm[D];       // g_q * g_k, read as float4 slices
@@ -112,29 +115,45 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   // every wave-wide load would touch 32 cache lines for 32 bytes each and the prologue would spend its time in
   // the address path of the vector memory unit; staged through LDS by direct loads they are whole lines, and the
   // row-major fragment read of a tile is exactly the B-operand layout (lane = row, 8 entries of k-step ks).
-  // Stage 0 takes key tile 0; stages 1..3 hold the q, dO and o blocks until the rows sit in registers, then
-  // key tiles 1 and 2 are requested into stages 1 and 2 and the ring turns as usual.  All of it is in flight at
-  // once, with the row's lse, the gate logit and the scale vector behind it: one memory round trip (vector-memory
-  // waits are in order, and the compiler's own count does not see the direct loads, so its first wait covers
-  // them).  The prologue's results (Qhat, gated dO, -delta, -lse2, dgate) are stored from the epilogue, so no
-  // store is in flight while the loop counts its tile loads.
+  // Without a rotary embedding: stage 0 takes key tile 0; stages 1..3 hold the q, dO and o blocks until the rows sit
+  // in registers, then key tiles 1 and 2 are requested into stages 1 and 2 and the ring turns as usual.  All of it
+  // is in flight at once, with the row's lse, the gate logit and the scale vector behind it: one memory round trip
+  // (vector-memory waits are in order, and the compiler's own count does not see the direct loads, so its first
+  // wait covers them).
+  // With a rotary embedding the table rows of the 128 positions (D/2 floats: as long as a tensor row) are two more
+  // blocks, for the same reason, and the start-up has two phases: q, cos, sin, dO in stages 0..3; once they are in
+  // registers, the o block in stage 3 and key tiles 0..2 in stages 0..2, which arrive while Qhat is computed.
+  // The prologue's results (Qhat, gated dO, -delta, -lse2, dgate) are stored from the epilogue, so no store is in
+  // flight while the loop counts its tile loads.
+  constexpr int kRowStage = R.row_stage_first;
+  constexpr int kQStage = ROPE ? 0 : kRowStage, kCosStage = 1, kSinStage = 2;
+  constexpr int kDoStage = ROPE ? 3 : kRowStage + 1, kOStage = ROPE ? kRowStage : kRowStage + 2;
+  static_assert(!ROPE || kOStage == 3, "first phase: q, cos, sin, dO; second phase: tiles 0..2, o");
+  const int rows_left = p.Sq - q0;
+  const char* qb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.q, b, h, q0));
+  const char* db = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, q0));
+  const char* yb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.o, b, h, q0));
+  const int64_t rope_row0 = ROPE ? (int64_t)(p.rope_q_pos0 + q0) * (D / 2) : 0;  // the tables' row of query q0
+  auto issue_rope_rows = [&](int cos_stage, int sin_stage) {  // 128 table rows each, laid out like tensor rows
+    const TileLaneOff<D> o = rowblock_lane_offsets<D>(D * 2, 0, rows_left, src.x, src.y);
+    const char* cb = reinterpret_cast<const char*>(p.rope_cos + rope_row0);
+    const char* sb = reinterpret_cast<const char*>(p.rope_sin + rope_row0);
+    issue_tile_pair<D>(cb, cb, o, wave_dst + cos_stage * kStageBytes);
+    issue_tile_pair<D>(sb, sb, o, wave_dst + sin_stage * kStageBytes);
+  };
+  if constexpr (ROPE) {
+    issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + kQStage * kStageBytes);
+    issue_rope_rows(kCosStage, kSinStage);
+    issue_tile_pair<D>(db, db, rowblock_lane_offsets<D>((uint32_t)p.d_o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + kDoStage * kStageBytes);
+  } else {
 #pragma unroll
-  for (int t = 0; t < R.early_tiles; ++t)
-    if (t < n_kt) issue_tile(t);
-  constexpr int kRowStage = R.row_stage_first;  // q, dO, o blocks in stages kRowStage, +1, +2
-  {
-    const int rows_left = p.Sq - q0;
-    const char* qb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.q, b, h, q0));
-    const char* db = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.d_o, b, h, q0));
-    const char* yb = reinterpret_cast<const char*>(row_ptr<uint16_t>(p.o, b, h, q0));
-    issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + kRowStage * kStageBytes);
-    issue_tile_pair<D>(db, db, rowblock_lane_offsets<D>((uint32_t)p.d_o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + (kRowStage + 1) * kStageBytes);
-    issue_tile_pair<D>(yb, yb, rowblock_lane_offsets<D>((uint32_t)p.o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + (kRowStage + 2) * kStageBytes);
+    for (int t = 0; t < R.early_tiles; ++t)
+      if (t < n_kt) issue_tile(t);
+    issue_tile_pair<D>(qb, qb, rowblock_lane_offsets<D>((uint32_t)p.q.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + kQStage * kStageBytes);
+    issue_tile_pair<D>(db, db, rowblock_lane_offsets<D>((uint32_t)p.d_o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + kDoStage * kStageBytes);
+    issue_tile_pair<D>(yb, yb, rowblock_lane_offsets<D>((uint32_t)p.o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + kOStage * kStageBytes);
   }
   const float lse_row = p.lse[ridx];
-  const int64_t rope_pos = ROPE ? (int64_t)(p.rope_q_pos0 + row_c) * (D / 2) : 0;
-  RopeB<KS> rope_b;
-  if (ROPE) rope_b = rope_b_load<KS>(p.rope_cos + rope_pos, p.rope_sin + rope_pos, hh);
   // the conditional reads last: the compiler waits for every outstanding load where their branches join
   float gate_z = 0.f;
   if (p.gate.ptr)
@@ -147,35 +166,54 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   // rows 32*wave .. 32*wave+31 of the block: half (wave >> 1) of each stage, row block (wave & 1) of that tile
   u32x4 qraw[KS], dyraw[KS], yraw[KS];
   u32x2 qct[MB][4];  // the query row once more, in the layout of the epilogue's C tiles (packed pairs)
+  RopeB<KS> rope_b;
+  const uint32_t row_half = (wave >> 1) * Z::kTileBytes, row_rb = wave & 1;
+  const uint32_t row_rm = lds0 + row_half + swz_off_rm<D>(lane);
+  const uint32_t row16 = lds0 + row_half + swz_off_row16<D>(lane) + row_rb * 32 * Z::kRB;  // chunk 0 of the lane's row
   {
-    const uint32_t half = (wave >> 1) * Z::kTileBytes, rb = wave & 1;
-    const uint32_t rm = lds0 + half + swz_off_rm<D>(lane);
-    const uint32_t ct = lds0 + kRowStage * kStageBytes + half + swz_off_ct<D>(lane) + rb * 32 * Z::kRB;
+    const uint32_t ct = lds0 + kQStage * kStageBytes + row_half + swz_off_ct<D>(lane) + row_rb * 32 * Z::kRB;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      qraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + kRowStage * kStageBytes, rb, ks));
-      dyraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + (kRowStage + 1) * kStageBytes, rb, ks));
-      yraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(rm + (kRowStage + 2) * kStageBytes, rb, ks));
+      qraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(row_rm + kQStage * kStageBytes, row_rb, ks));
+      dyraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(row_rm + kDoStage * kStageBytes, row_rb, ks));
+      if constexpr (!ROPE) yraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(row_rm + kOStage * kStageBytes, row_rb, ks));
     }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int c = 0; c < 4; ++c) qct[mb][c] = lds_read8(ct ^ (uint32_t)((4 * mb + c) << 4));
+    if constexpr (ROPE) rope_b = rope_b_from_lds<KS>(row16 + kCosStage * kStageBytes, row16 + kSinStage * kStageBytes, hh);
   }
   __syncthreads();  // the borrowed stages are free again
+  if constexpr (ROPE) {
+    issue_tile_pair<D>(yb, yb, rowblock_lane_offsets<D>((uint32_t)p.o.stride_s * 2, 0, rows_left, src.x, src.y), wave_dst + kOStage * kStageBytes);
 #pragma unroll
-  for (int t = R.early_tiles; t < R.startup_tiles; ++t)
-    if (t < n_kt) issue_tile(t);
+    for (int t = 0; t < R.early_tiles; ++t)
+      if (t < n_kt) issue_tile(t);
+  } else {
+#pragma unroll
+    for (int t = R.early_tiles; t < R.startup_tiles; ++t)
+      if (t < n_kt) issue_tile(t);
+  }
 
   // ---- query-row prologue: alpha, Qhat, delta, gate; B operands stay in registers
   bf16x8 qreg[KS], doreg[KS];
-  float alpha, delta, dgate_row = 0.f, gfac = 1.f;
-  {
+  float alpha, delta, dgate_row = 0.f, gfac = 1.f, gate_sg = 0.f;
+  auto row_dot = [&]() {  // delta = rowsum(dY * Y): the o block is the last thing the second phase waits for
     float dl = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int i = 0; i < 4; ++i) dl += bf16lo(yraw[ks][i]) * bf16lo(dyraw[ks][i]) + bf16hi(yraw[ks][i]) * bf16hi(dyraw[ks][i]);
+    delta = half_sum(dl);
+    if (p.gate.ptr) dgate_row = (1.0f - gate_sg) * delta;
+  };
+  if (p.gate.ptr) {
+    gate_sg = 1.0f / (1.0f + __expf(-gate_z));
+    gfac = p.gate_scale * gate_sg;
+  }
+  if constexpr (!ROPE) row_dot();
+  {
     float qx[KS][8];
     unpack_b_layout<KS>(qraw, qx);
     if (ROPE) rope_b_apply<KS>(qx, rope_b);
@@ -185,14 +223,8 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
 #pragma unroll
       for (int t = 0; t < 8; ++t) ss += qx[ks][t] * qx[ks][t];
     ss = half_sum(ss);
-    delta = half_sum(dl);
     alpha = row_normaliser_fast(p, ss, 1.0f / D);
     const float f = alpha * p.sm_scale * kLog2e;
-    if (p.gate.ptr) {
-      const float sg = 1.0f / (1.0f + __expf(-gate_z));
-      gfac = p.gate_scale * sg;
-      dgate_row = (1.0f - sg) * delta;
-    }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const float4 ga = *reinterpret_cast<const float4*>(gsm + 16 * ks + 8 * hh);
@@ -205,6 +237,16 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
       qreg[ks] = as_bf16x8(w);
       doreg[ks] = as_bf16x8(p.gate.ptr ? scale8(dyraw[ks], gfac) : dyraw[ks]);
     }
+  }
+  if constexpr (ROPE) {
+    // second phase landed (tile 2 with it: no late tile, no further wait before the loop); the o rows go to registers
+    // and one more barrier frees their stage, which iteration 0 refills
+    wait_vmcnt<0>();
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) yraw[ks] = __builtin_bit_cast(u32x4, swz_frag_rm<D>(row_rm + kOStage * kStageBytes, row_rb, ks));
+    row_dot();
+    __syncthreads();
   }
   // row statistics as MFMA C operands (every register of a lane belongs to the lane's query); the dK/dV
   // kernel reads the same two numbers per row from the workspace
@@ -270,8 +312,10 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   // second block of a tile already requests the next tile's fragments) and at most one more in flight, so tile 1,
   // requested after the row blocks had left its stage, must be complete here; the row prologue above ran in
   // between, so this wait is short.  Tile 2 stays in flight.
-  if (n_kt >= R.startup_tiles) wait_vmcnt<ring::loads_kept_before_loop(R, R.startup_tiles)>(); else wait_vmcnt<0>();
-  __syncthreads();
+  if constexpr (R.wait_before_loop) {
+    if (n_kt >= R.startup_tiles) wait_vmcnt<ring::loads_kept_before_loop(R, R.startup_tiles)>(); else wait_vmcnt<0>();
+    __syncthreads();
+  }
   if (n_act > 0) request_rowmajor(rm_lane, 0);
   // leading blocks of this wave that need no mask (every key visible to every query of the wave, inside Sk)
   int n_full = p.Sk / 32;
@@ -305,8 +349,17 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   // f > 0 reaches that kernel through the two statistics and it streams the caller's dO as it is: with
   // P' = f P = exp2(S - lse2 + log2 f) it holds dV' = P'^T dO and dS = P (f dP - delta) = P' (dP - delta / f).  A
   // factor that underflowed switches the row off (P' = 0).  Only a gate scale <= 0 needs the gated copy of dO.
+  // With a rotary embedding the table rows come in once more, into the idle ring (every wave has passed the last
+  // iteration's barrier), now for the accumulators' layout; the second barrier keeps the scale-gradient staging
+  // below, which reuses the ring, behind every wave's reads.
   RopeCt<MB> rope_ct;
-  if (ROPE) rope_ct = rope_ct_load<MB>(p.rope_cos + rope_pos, p.rope_sin + rope_pos, hh);
+  if constexpr (ROPE) {
+    issue_rope_rows(0, 1);
+    wait_vmcnt<0>();
+    __syncthreads();
+    rope_ct = rope_ct_from_lds<MB>(row16, row16 + kStageBytes, hh);
+    __syncthreads();
+  }
   if (live) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -638,6 +691,7 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dkdv_bf16_kern
   // passed the last iteration's barrier), and from there in the accumulators' layout.  Read row-per-lane from global
   // memory, 8 bytes per lane, every wave-wide load would touch 32 cache lines and the three tensors would keep the
   // address path of the vector memory unit busy for 4-12 us of the launch.
+  static_assert(R.epilogue_row_stages == 3, "k, v, v_first blocks in stages 0, 1, 2");
   const bool live = key < p.Sk;
   float c1 = 1.f, c2 = 0.f;
   if (p.vr_coef) { c1 = p.vr_coef[0]; c2 = p.vr_coef[1]; }

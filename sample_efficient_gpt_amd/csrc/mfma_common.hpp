@@ -390,6 +390,44 @@ __device__ __forceinline__ int swz_off_ct(int lane) {
 __device__ __forceinline__ u32x2 lds_read8(uint32_t addr) {
   return *(const __attribute__((address_space(3))) u32x2*)addr;
 }
+// Per-lane byte offset (within a tile) of chunk 0 of the lane's row (row l%32 of a 32-row block): the 16-byte chunk
+// c of that row is at this offset XOR (c << 4); row block rb adds 32*kRB.
+template <int D>
+__device__ __forceinline__ int swz_off_row16(int lane) {
+  const int ln = lane & 31;
+  return ln * Swz<D>::kRB + (Swz<D>::f(ln) << 4);
+}
+// Rotary table rows staged in LDS as row blocks: a table row (D/2 floats) is as long as a bf16 tensor row (kRB bytes),
+// so the 128 positions of a workgroup travel and are laid out exactly like 128 tensor rows.  cos16 / sin16: LDS
+// address of chunk 0 of the lane's row in either block.  Same register contents as rope_b_load / rope_ct_load.
+template <int KS>
+__device__ __forceinline__ RopeB<KS> rope_b_from_lds(uint32_t cos16, uint32_t sin16, int hh) {
+  RopeB<KS> r;
+#pragma unroll
+  for (int ks = 0; ks < KS / 2; ++ks)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t off = (uint32_t)((4 * ks + 2 * hh + j) << 4);  // floats 16 ks + 8 hh + 4 j ..
+      const f32x4 c = lds_read_f4(cos16 ^ off), sn = lds_read_f4(sin16 ^ off);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { r.c[ks][4 * j + i] = c[i]; r.s[ks][4 * j + i] = sn[i]; }
+    }
+  return r;
+}
+template <int MB>
+__device__ __forceinline__ RopeCt<MB> rope_ct_from_lds(uint32_t cos16, uint32_t sin16, int hh) {
+  RopeCt<MB> r;
+#pragma unroll
+  for (int mb = 0; mb < MB / 2; ++mb)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint32_t off = (uint32_t)((8 * mb + 2 * c + hh) << 4);  // floats 32 mb + 8 c + 4 hh ..
+      const f32x4 cs = lds_read_f4(cos16 ^ off), sn = lds_read_f4(sin16 ^ off);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { r.c[mb][4 * c + i] = cs[i]; r.s[mb][4 * c + i] = sn[i]; }
+    }
+  return r;
+}
 //   src_a/src_b: wave-uniform pointers to row `row0` of each tensor; dst: LDS byte address of the stage + wave*1024
 template <int D, int ROWS = kBK>
 __device__ __forceinline__ void issue_tile_pair(const char* src_a, const char* src_b, const TileLaneOff<D, ROWS>& o, uint32_t dst) {

@@ -30,6 +30,12 @@ struct Protocol {
   int issue_ahead;       // ... namely tile jt + issue_ahead, into the stage that tile jt-1 has just left
   int keep_tiles;        // the wait that ends an iteration which requested a tile leaves this many of the youngest
                          // tiles in flight (an iteration that requested none waits for everything)
+  int pre_row_stages = 0;   // a start-up phase of its own BEFORE all of the above: row blocks in stages
+                            // [0, pre_row_stages), awaited, read into registers, one barrier; then the stages are free
+  int epilogue_row_stages = 0;  // behind the loop (the ring is idle: every wave has passed the last iteration's
+                            // barrier) up to this many row blocks for the epilogue are requested into stages
+                            // [0, epilogue_row_stages), awaited, published by one barrier and read into registers
+  bool epilogue_reuses_ring = false;  // the epilogue afterwards writes scratch data over the ring's stages
 };
 
 // An iteration needs its own tile and the next one landed.
@@ -55,15 +61,21 @@ constexpr Protocol forward(int stages, int q_stages, int passes) {
 }
 // dQ: key tile 0 in stage 0, the q / dO / o row blocks in stages 1..3, then key tiles 1 and 2; tile 1 is a late
 // request, hence the wait before the loop.
-constexpr Protocol dq(int passes) { return Protocol{4, 2 * passes, 1, 1, 3, 3, true, false, 3, 1}; }
+constexpr Protocol dq(int passes) { return Protocol{4, 2 * passes, 1, 1, 3, 3, true, false, 3, 1, 0, 0, true}; }
+// dQ with a rotary embedding: the table rows of the workgroup's 128 positions are row blocks too.  First phase: q,
+// cos, sin, dO in stages 0..3; second phase: key tiles 0..2 in stages 0..2 and the o block in stage 3 (everything
+// awaited: no late tiles).  The cos and sin blocks come once more behind the loop, for the epilogue.
+constexpr Protocol dq_rope(int passes) { return Protocol{4, 2 * passes, 3, 3, 1, 3, false, false, 3, 1, 4, 2, true}; }
 // dK/dV: (Qhat, dO) tiles 0 and 1 in stages 0 and 1 with the Khat / V' row blocks in stages 2 and 3, then tile 2;
 // a tile is the two [64, D] tiles plus one row-statistics load.
-constexpr Protocol dkdv(int passes) { return Protocol{4, 2 * passes + 1, 2, 2, 2, 3, false, false, 3, 1}; }
+// Behind the loop: the raw k block (and, with a value residual, the raw v and v_first blocks) for the epilogue.
+constexpr Protocol dkdv(int passes) { return Protocol{4, 2 * passes + 1, 2, 2, 2, 3, false, false, 3, 1, 0, 3, false}; }
 
 constexpr bool well_formed(const Protocol& p) {
   return p.stages >= 3 && p.early_tiles >= 1 && p.early_tiles <= p.startup_tiles && p.startup_tiles <= p.stages - 1 &&
          p.row_stage_first >= p.early_tiles && p.row_stage_first + p.row_stages <= p.stages && p.keep_tiles >= 0 &&
-         p.issue_ahead >= kTilesNeededAtLoopStart;
+         p.issue_ahead >= kTilesNeededAtLoopStart && p.pre_row_stages >= 0 && p.pre_row_stages <= p.stages &&
+         p.epilogue_row_stages >= 0 && p.epilogue_row_stages <= p.stages;
 }
 
 }  // namespace ring

@@ -29,19 +29,29 @@ enum Kind { REQUEST, WAIT, BARRIER, READ };
 struct Op {
   Kind kind;
   int stage;    // REQUEST / READ
-  int content;  // REQUEST / READ: tile index >= 0, or kRows
-  int n;        // REQUEST: loads issued by the wave; WAIT: the vmcnt immediate
+  int content;  // REQUEST / READ: tile index >= 0, kRows, kPreRows, kEpilogueRows or kScratch
+  int n;        // REQUEST: loads issued by the wave (0: plain LDS stores, e.g. the epilogue's scratch); WAIT: the vmcnt immediate
 };
-constexpr int kRows = -1;
+constexpr int kRows = -1, kPreRows = -3, kEpilogueRows = -5, kScratch = -4;
 
 // The order of operations of one wave, following fwd_mfma.hip / bwd_mfma.hip:
+//   [first start-up phase: row blocks in stages 0 .., wait for everything, barrier, rows -> registers, barrier;]
 //   start-up: early tiles, row blocks, wait for everything, barrier, rows -> registers, barrier, late tiles,
 //             [wait + barrier], fragment request of tile 0;
 //   iteration jt: [request at top], blocks of tile jt (its stage; the second block also requests the row-major
-//             fragments of tile jt+1 from the NEXT stage), [request at bottom], wait, barrier.
-std::vector<Op> wave_program(const Protocol& p, int n_tiles, int row_loads_per_stage) {
+//             fragments of tile jt+1 from the NEXT stage), [request at bottom], wait, barrier;
+//   [behind the loop: `epilogue_rows` row blocks (at most p.epilogue_row_stages) requested into stages 0 .., wait for
+//    everything, barrier, rows -> registers, barrier, scratch stores over the ring].
+std::vector<Op> wave_program(const Protocol& p, int n_tiles, int row_loads_per_stage, int epilogue_rows = 0) {
   std::vector<Op> ops;
   auto request_tile = [&](int t) { ops.push_back({REQUEST, t % p.stages, t, p.loads_per_tile}); };
+  if (p.pre_row_stages > 0) {
+    for (int i = 0; i < p.pre_row_stages; ++i) ops.push_back({REQUEST, i, kPreRows, row_loads_per_stage});
+    ops.push_back({WAIT, 0, 0, 0});
+    ops.push_back({BARRIER, 0, 0, 0});
+    for (int i = 0; i < p.pre_row_stages; ++i) ops.push_back({READ, i, kPreRows, 0});
+    ops.push_back({BARRIER, 0, 0, 0});
+  }
   for (int t = 0; t < p.early_tiles; ++t)
     if (t < n_tiles) request_tile(t);
   for (int i = 0; i < p.row_stages; ++i) ops.push_back({REQUEST, p.row_stage_first + i, kRows, row_loads_per_stage});
@@ -60,12 +70,21 @@ std::vector<Op> wave_program(const Protocol& p, int n_tiles, int row_loads_per_s
   for (int jt = 0; jt < n_tiles; ++jt) {
     const bool requested = jt + p.issue_ahead < n_tiles;
     if (p.issue_at_top && requested) request_tile(jt + p.issue_ahead);
-    ops.push_back({READ, jt % p.stages, jt, 0});                                    // both blocks, both orientations
-    if (jt + 1 < n_tiles) ops.push_back({READ, (jt + 1) % p.stages, jt + 1, 0});    // next tile's first fragments
+    ops.push_back({READ, jt % p.stages, jt, 0});                                      // both blocks, both orientations
+    if (jt + 1 < n_tiles) ops.push_back({READ, (jt + 1) % p.stages, jt + 1, 0});      // next tile's first fragments
     if (!p.issue_at_top && requested) request_tile(jt + p.issue_ahead);
     ops.push_back({WAIT, 0, 0, segpt::ring::loads_kept_after_iteration(p, requested)});
     ops.push_back({BARRIER, 0, 0, 0});
   }
+  if (epilogue_rows > 0) {
+    for (int i = 0; i < epilogue_rows; ++i) ops.push_back({REQUEST, i, kEpilogueRows, row_loads_per_stage});
+    ops.push_back({WAIT, 0, 0, 0});
+    ops.push_back({BARRIER, 0, 0, 0});
+    for (int i = 0; i < epilogue_rows; ++i) ops.push_back({READ, i, kEpilogueRows, 0});
+    if (p.epilogue_reuses_ring) ops.push_back({BARRIER, 0, 0, 0});
+  }
+  if (p.epilogue_reuses_ring)
+    for (int i = 0; i < p.stages; ++i) ops.push_back({REQUEST, i, kScratch, 0});
   return ops;
 }
 
@@ -93,7 +112,7 @@ std::string replay(const Protocol& p, const std::vector<Op>& ops) {
             return buf;
           }
         }
-        s.content = o.content; s.loads_pending = o.n; s.retired_epoch = -1; s.last_read_epoch = -1; s.ever = true;
+        s.content = o.content; s.loads_pending = o.n; s.retired_epoch = o.n == 0 ? epoch : -1; s.last_read_epoch = -1; s.ever = true;
         for (int k = 0; k < o.n; ++k) queue.push_back({o.stage, o.content});
         break;
       }
@@ -126,12 +145,14 @@ std::string replay(const Protocol& p, const std::vector<Op>& ops) {
   return "";
 }
 
-std::string check(const Protocol& p, int max_tiles) {
+// every streamed-tile count from min_tiles on, with every count of epilogue row blocks the protocol allows
+std::string check(const Protocol& p, int max_tiles, int min_tiles = 1) {
   if (!segpt::ring::well_formed(p)) return "not well formed";
-  for (int n = 1; n <= max_tiles; ++n) {
-    const std::string v = replay(p, wave_program(p, n, 2 * p.loads_per_tile));
-    if (!v.empty()) return "n_tiles " + std::to_string(n) + ": " + v;
-  }
+  for (int rows = 0; rows <= p.epilogue_row_stages; ++rows)
+    for (int n = min_tiles; n <= max_tiles; ++n) {
+      const std::string v = replay(p, wave_program(p, n, 2 * p.loads_per_tile, rows));
+      if (!v.empty()) return "n_tiles " + std::to_string(n) + " + " + std::to_string(rows) + " epilogue row blocks: " + v;
+    }
   return "";
 }
 
@@ -147,10 +168,12 @@ int main() {
         {"forward, 32 rows per wave (3 stages; head_dim 64 up to 2048 keys, head_dim 128)", forward(3, 1, passes)},
         {"forward, 64 rows per wave (4 stages; head_dim 64 beyond 2048 keys)", forward(4, 2, passes)},
         {"dQ", dq(passes)},
-        {"dK/dV", dkdv(passes)},
+        {"dQ with a rotary embedding (two start-up phases, table rows once more behind the loop)", dq_rope(passes)},
+        {"dK/dV (k, v, v_first rows behind the loop; a key tile may see no query at all)", dkdv(passes)},
     };
     for (const Named& k : shipped) {
-      const std::string v = check(k.p, 70);
+      const bool can_be_empty = k.p.loads_per_tile == 2 * passes + 1;  // dK/dV: key tiles beyond every query
+      const std::string v = check(k.p, 70, can_be_empty ? 0 : 1);
       printf("passes %d  %-82s %s\n", passes, k.name, v.empty() ? "ok" : ("VIOLATION: " + v).c_str());
       failures += !v.empty();
     }
@@ -192,6 +215,34 @@ int main() {
       if (o.kind == REQUEST && o.content >= 0) o.n = p.loads_per_tile - 1;
     const std::string v = replay(p, ops);
     printf("%-82s %s\n", "dK/dV counting five loads per tile while issuing four", v.empty() ? "NOT CAUGHT" : ("caught: " + v).c_str());
+    failures += v.empty();
+  }
+  // ---- the row blocks around the loop, broken by leaving out one barrier or wait of the generated order
+  auto drop = [](std::vector<Op> ops, Kind kind, int which_from_end) {  // removes the which-th last op of a kind
+    for (int i = (int)ops.size() - 1; i >= 0; --i)
+      if (ops[i].kind == kind && which_from_end-- == 0) { ops.erase(ops.begin() + i); break; }
+    return ops;
+  };
+  auto drop_nth = [](std::vector<Op> ops, Kind kind, int which) {        // removes the which-th op of a kind
+    for (size_t i = 0; i < ops.size(); ++i)
+      if (ops[i].kind == kind && which-- == 0) { ops.erase(ops.begin() + i); break; }
+    return ops;
+  };
+  struct BrokenOps { const char* name; Protocol p; std::vector<Op> ops; };
+  const Protocol dr = dq_rope(passes), dk = dkdv(passes);
+  const BrokenOps broken_ops[] = {
+      {"dK/dV reading its epilogue row blocks without the wait behind their requests", dk,
+       drop(wave_program(dk, 12, 2 * dk.loads_per_tile, 3), WAIT, 0)},
+      {"dK/dV reading its epilogue row blocks without the barrier behind the wait", dk,
+       drop(wave_program(dk, 12, 2 * dk.loads_per_tile, 3), BARRIER, 0)},
+      {"dQ (rotary) requesting the second start-up phase without the barrier behind the first phase's reads", dr,
+       drop_nth(wave_program(dr, 12, 2 * dr.loads_per_tile, 2), BARRIER, 1)},
+      {"dQ (rotary) writing the epilogue's scratch over the ring without a barrier behind the table-row reads", dr,
+       drop(wave_program(dr, 12, 2 * dr.loads_per_tile, 2), BARRIER, 0)},
+  };
+  for (const BrokenOps& k : broken_ops) {
+    const std::string v = replay(k.p, k.ops);
+    printf("%-104s %s\n", k.name, v.empty() ? "NOT CAUGHT" : ("caught: " + v).c_str());
     failures += v.empty();
   }
   return failures ? 1 : 0;

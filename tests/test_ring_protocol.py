@@ -36,10 +36,10 @@ def test_shipped_protocols_hold_and_broken_ones_are_caught(checker):
     assert proc.returncode == 0, out
     lines = out.strip().splitlines()
     ok = [l for l in lines if l.rstrip().endswith(" ok")]
-    assert len(ok) == 8, out  # four kernels' pipelines at both head dims
+    assert len(ok) == 10, out  # five pipelines (forward 2 shapes, dQ, dQ with rotary tables, dK/dV) at both head dims
     assert "VIOLATION" not in out and "NOT CAUGHT" not in out, out
     caught = [l for l in lines if "caught:" in l]
-    assert len(caught) == 5, out
+    assert len(caught) == 9, out
     # the start-up bug that once shipped must be reported as exactly what it was
     bug = next(l for l in caught if l.startswith("dQ without the wait before the loop"))
     assert "read of content 1" in bug and "before it has landed" in bug, bug
