@@ -109,6 +109,8 @@ def test_fp32_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
         (1, 2, 2, 128, 128, 64, {"eps": 1e-8 / 64, "sm_scale": 1 / 64}, {"scalar_gain": True, "no_gk": True}),
         (2, 4, 2, 300, 130, 64, {}, {}),               # causal with more queries than keys: rows >= 130 see every key
         (1, 2, 1, 257, 64, 128, {}, {"extras": True}),
+        (1, 2, 1, 100, 400, 64, {"gate_scale": 2.0}, {"extras": True}),  # key tiles beyond every query: dK/dV workgroups without a loop
+        (1, 2, 2, 60, 300, 128, {}, {}),
     ],
 )
 def test_bf16_fwd_bwd(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
@@ -501,6 +503,16 @@ def test_positional_dropin_functions_under_torch_compile(gpu_device):
         (1, 3, 3, 72, 200, 64, {"q_start": 128}, {}),                      # queries at positions 128.. (attention.py:191-195)
         (1, 2, 1, 96, 96, 64, {"rope_q_pos0": 40, "rope_k_pos0": 40}, {}),  # explicit positions
         (1, 2, 2, 80, 140, 64, {"causal": False}, {}),
+        # the dQ kernel's two-phase start-up with one, two and three key tiles in all (its second phase requests up to
+        # three), and a last query block of 5 rows (the staged table blocks repeat the last row)
+        (2, 2, 1, 40, 40, 64, {"gate_scale": 2.0}, {"extras": True}),
+        (1, 4, 2, 100, 100, 64, {}, {}),
+        (1, 2, 2, 133, 133, 64, {"gate_scale": 2.0}, {"extras": True}),
+        (1, 4, 1, 333, 333, 128, {"gate_scale": 2.0}, {"extras": True}),
+        # key tiles beyond every query (causal, fewer queries than keys, no offset): the dK/dV workgroups of those
+        # tiles stream nothing and go straight to the epilogue's row blocks; their dk, dv are zero
+        (1, 2, 1, 100, 400, 64, {"gate_scale": 2.0}, {"extras": True}),
+        (1, 2, 1, 70, 300, 128, {}, {}),
     ],
 )
 def test_bf16_fused_rope(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
@@ -509,6 +521,15 @@ def test_bf16_fused_rope(gpu_device, B, H, Hkv, Sq, Sk, D, kw, gen_kw):
     gradients by autograd (fp64)."""
     cos, sin = orc.rope_tables(512, 10000.0, D)
     _case(gpu_device, BF16, B, H, Hkv, Sq, Sk, D, gen_kw=gen_kw, seed=31, rope=(cos, sin), **kw)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_bf16_fused_rope_tables_of_exactly_the_needed_length(gpu_device, D):
+    """Tables with exactly as many rows as there are positions (the staged table blocks of the last, partial query
+    block must stay inside them), with positions offset into the tables for q."""
+    Sq, Sk = 77, 205
+    cos, sin = orc.rope_tables(Sk, 10000.0, D)
+    _case(gpu_device, BF16, 1, 4, 2, Sq, Sk, D, gen_kw={"extras": True}, seed=33, rope=(cos, sin), gate_scale=2.0, q_start=Sk - Sq)
 
 
 def test_fused_rope_equals_rotating_first_and_rejects_bad_tables(gpu_device):
