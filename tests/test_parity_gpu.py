@@ -1334,6 +1334,35 @@ def test_full_size_steps_repeat_bit_for_bit(gpu_device, B, S, steps):
             assert torch.equal(a, b), f"step {it}: {name} differs from the first step"
 
 
+@pytest.mark.parametrize("B,S,steps", [(8, 2048, 50), (21, 768, 200), (3, 1100, 200)])
+def test_module_shaped_steps_repeat_bit_for_bit(gpu_device, B, S, steps):
+    """The same on the call the attention module makes (strided views of one projection buffer, rotary embedding,
+    scalar gain, gate, value residual): its kernels have start-up and epilogue phases of their own (the dQ kernel's
+    two-phase start-up with the rotary table blocks, the row blocks behind the loops of dQ and dK/dV, the gate
+    factor inside the row statistics); S = 1100 leaves a last query block of 76 rows."""
+    import bench
+    from sample_efficient_gpt_amd.plan import AttnPlan
+
+    c = CONFIGS[3].scaled(extras=True, B=B, S=S)
+    x, rope = bench.module_shaped_inputs(c, gpu_device)
+    plan = AttnPlan(x, eps=c.eps, sm_scale=c.sm_scale, gate_scale=2.0, backward=True, rope_cos=rope[0], rope_sin=rope[1],
+                    rope_q_pos0=0, rope_k_pos0=0)
+    names = ("y", "lse", "dq", "dk", "dv", "dv_first", "dgate", "dg_q", "dcoef")
+    outs = [getattr(plan, n) for n in names]
+    plan.forward()
+    plan.backward(kv_prepared=True)
+    torch.cuda.synchronize()
+    ref = [t.clone() for t in outs]
+    print(f"module-shaped repeatability B={B} S={S}", flush=True)
+    for it in range(steps):
+        for t in outs[:7]:
+            t.zero_()
+        plan.forward()
+        plan.backward(kv_prepared=True)
+        for name, a, b in zip(names, outs, ref):
+            assert torch.equal(a, b), f"step {it}: {name} differs from the first step"
+
+
 def test_empty_batch_and_no_query_rows(gpu_device):
     """B = 0 and Sq = 0: empty outputs, zero gradients, nothing launched (like torch's SDPA on empty inputs)."""
     d = gpu_device
