@@ -278,6 +278,18 @@ __global__ __launch_bounds__(kThreadsM, D == 64 ? 2 : 1) void bwd_dq_bf16_kernel
   // MASKED is compile-time so that a whole block is one straight-line scheduling region
   auto step = [&](auto masked_c, uint32_t tr, int kb, int jb, uint32_t next_rm, int next_kb) {
     constexpr bool MASKED = decltype(masked_c)::value != 0;
+    // head_dim 128 runs one wave per SIMD with all 256 ordinary registers in use: left to itself the compiler requests
+    // each LDS fragment one MFMA ahead of its use and the wave stalls on LDS latency before most MFMAs.  Asking for
+    // the block as 24 groups of (1 MFMA, 2 LDS reads, 2 vector instructions) keeps two requests ahead: -6 % on this
+    // kernel (neighbouring group shapes are 2-10 % slower; at head_dim 64, two waves per SIMD, none changes anything).
+    if constexpr (D == 128) {
+#pragma unroll
+      for (int i = 0; i < 3 * KS; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS read
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // VALU
+      }
+    }
     f32x16 s = c_lse, dpv = c_del;
     // the S chain first, then the dP chain: exp2 of the finished scores runs behind the dP MFMAs
 #pragma unroll
